@@ -521,10 +521,10 @@ int mi355_add_layernorm_fwd(int64_t tokens, int width, const float* x, float alp
 /* out[t, :n] = x[t, :n] / sqrt(mean(x[t, :n]^2) + eps) * w on strided rows. */
 int mi355_rmsnorm_rows(int64_t tokens, int n, const void* x, int x_dt, int64_t ldx, const float* w, float eps, void* out, int out_dt, int64_t ldo,
                        void* stream);
-/* Latent key/value rows: src[t] = [rank | rot] values; cache row dst_row[t] <- [RMSNorm(first rank) * w | last rot with the pairs (2i, 2i+1), 2i+1 < dims,
- * turned by pos[t] * freq[i]]. */
+/* Latent key/value rows: src[t] = [rank | rot] values; cache row dst_row[t] <- [RMSNorm(first rank) * w | last rot with its first `dims` entries turned by
+ * pos[t] * freq[i]]: layout 0 pairs the entries (2i, 2i+1), layout 1 the entries (i, i + dims/2). */
 int mi355_latent_kv_append(int64_t tokens, int rank, int rot, const void* src, int src_dt, int64_t ld, const float* w, float eps, const int* pos,
-                           const int* dst_row, const float* freq, int dims, void* cache, int cache_dt, int64_t ldc, void* stream);
+                           const int* dst_row, const float* freq, int dims, int layout, void* cache, int cache_dt, int64_t ldc, void* stream);
 /* dst[t, h * dst_hs + dst_off + i] = src[t, h * src_hs + src_off + i] for i < n (dst fp32), the pairs of [rot_start, rot_start + dims) turned by
  * pos[t] * freq[i].  layout 0: pair i = entries (2i, 2i+1) (interleaved rotary embedding); layout 1: pair i = entries (i, i + dims/2) (rotate-half). */
 int mi355_rope_heads(int64_t tokens, int H, int n, const void* src, int src_dt, int64_t ld_src, int src_hs, int src_off, float* dst, int64_t ld_dst,
@@ -564,11 +564,16 @@ int mi355_bgemm(int batch, int M, int N, int K, const void* A, int a_dt, int64_t
  * D1 + D2 <= 320, DV <= 256) 128 / hm tokens, and with splits > 1 deals a tile's keys to that many workgroups whose partial results meet in ws
  * (n_seq * head tiles * token tiles * splits * 128 * (2 + DV rounded up to 32 / 64 / 128 / 256) floats).
  * Grouped queries: head h reads key / value head h / kv_rep (strides k1_hs / v_hs per key / value head; hm may then divide kv_rep).  window > 0: the query
- * at position i sees key j <= i only if i - j < window or j < keep_first (a sliding window that keeps the first tokens); window 0: every j <= i. */
+ * at position i sees key j <= i only if i - j < window or j < keep_first (a sliding window that keeps the first tokens); window 0: every j <= i.
+ * softcap > 0: score <- softcap * tanh(score / softcap) after the scale.  sink (fp32 [H], may be NULL): exp(sink[h]) joins head h's softmax denominator.
+ * pool > 0 (needs window > 0, keep_first == 0, D2 == 0): besides the window the query at position i sees one pooled key / value row for every block b of
+ * `pool` tokens with (b + 1) * pool <= i - window + 1; block b of sequence s is row pool_row0[s] + b of PK / PV (pitch ldp, head strides k1_hs / v_hs,
+ * dtype dt); pooled rows and tokens share one softmax. */
 int mi355_latent_attn(int n_seq, int max_new, int H, int hm, int D1, int D2, int DV, const float* Q, int64_t ldq, int q_hs, const void* K1, int64_t ldk1,
                       int k1_hs, const void* K2, int64_t ldk2, const void* V, int64_t ldv, int v_hs, void* O, int64_t ldo, int o_hs, int dt,
                       const int* q_row0, const int* n_new, const int* past, const int* k1_row0, const int* k2_row0, const int* v_row0, float scale,
-                      int use_mfma, int splits, float* ws, int64_t ws_floats, int kv_rep, int window, int keep_first, void* stream);
+                      int use_mfma, int splits, float* ws, int64_t ws_floats, int kv_rep, int window, int keep_first, float softcap, const float* sink,
+                      int pool, const void* PK, const void* PV, int64_t ldp, const int* pool_row0, void* stream);
 
 /* ---- parallel-sublayer hybrid decoders in ragged batches (csrc/seqrec.hip) ---- */
 /* v = x + y1[t] + sum_{p < parts} y2[t * parts + p] (fp32 rows; y1 / y2 of dtype y*_dt, may be NULL); x_out (may be NULL or x) <- v.  For each weight
@@ -585,10 +590,13 @@ int mi355_ragged_conv(int64_t tokens, int n_seq, int C, int taps, const void* x,
                       const int* slot, float* state, int act, int residual, void* y, int y_dt, int64_t ldy, void* stream);
 /* Query / key / value rows of grouped-query attention: src[t] = [H x d | G x d | G x dv] (+ bias fp32, may be NULL); query and key heads get an RMS norm over d
  * (weights qw / kw fp32 [d], NULL: none) and a rotation of their first `dims` entries (layout as mi355_rope_heads); query head h times qscale[h] (may be NULL)
- * goes to q_out fp32 [t, h * d]; key and value heads go to cache row dst_row[t] = [G x d | G x dv] of dtype c_dt. */
+ * goes to q_out fp32 [t, h * d]; key and value heads go to cache row dst_row[t] = [G x d | G x dv] of dtype c_dt.  qt_every > 0: the query at position p
+ * is also multiplied by 1 + qt_coef * ln(floor((p + 1) / qt_every) + 1).  vmix (fp32 rows [G x dv], pitch ldvm, may be NULL): the cached value is
+ * (1 - lam) v + lam * vmix[t]. */
 int mi355_qkv_rows_append(int64_t tokens, int H, int G, int d, int dv, const void* src, int src_dt, int64_t ld_src, const float* bias, const float* qw,
                           const float* kw, float eps, const float* qscale, int dims, int layout, const float* freq, const int* pos, const int* dst_row,
-                          float* q_out, int64_t ldq, void* cache, int c_dt, int64_t ldc, void* stream);
+                          float* q_out, int64_t ldq, void* cache, int c_dt, int64_t ldc, float qt_coef, int qt_every, const float* vmix, int64_t ldvm, float lam,
+                          void* stream);
 /* Gated delta rule over the rows [seq_off[s], seq_off[s+1]) of each sequence, state[slot[s]] (fp32 [H, dk, dv]) read and written.  q / k rows [G * dk] (raw:
  * made unit vectors here, x / sqrt(sum x^2 + 1e-6), q also times qscale), v rows [H * dv]; value head h uses query / key head h / (H / G);
  * beta = sigmoid(b[t, h]), g = exp(-exp(A_log[h]) * softplus(a[t, h] + dt_bias[h])).  Per token: S <- g S; u = beta (v - S^T k); S <- S + k u^T; o = S^T q.
@@ -599,6 +607,20 @@ int mi355_delta_rule_ragged(int64_t tokens, int n_seq, const int* seq_off, const
 /* Gated feed-forward activation on rows [gate (F) | up (F)] -> [F].  kind 0: gelu_tanh(gate) * up.  kind 1: g = min(gate, limit), u = clamp(up, -limit, limit),
  * g * sigmoid(1.702 g) * (u + 1). */
 int mi355_glu_rows(int64_t rows, int F, const void* in, int in_dt, int64_t ld_in, int kind, float limit, void* out, int out_dt, int64_t ld_out, void* stream);
+
+/* ---- decoders with sandwich norms in ragged batches (csrc/seqsand.hip) ---- */
+/* v = x + y / sqrt(mean(y^2) + eps) * w_post (fp32 rows; y of dtype y_dt and pitch ldy, may be NULL: v = x); x_out (may be NULL or x) <- v;
+ * out (dtype out_dt, may be NULL together with w_next) <- v / sqrt(mean(v^2) + eps) * w_next.  width <= 8192. */
+int mi355_sandwich_rmsnorm(int64_t tokens, int width, const float* x, const void* y, int y_dt, int64_t ldy, const float* w_post, float* x_out,
+                           const float* w_next, float eps, void* out, int out_dt, void* stream);
+/* Mean rows of the blocks of `pool` cache rows that a step completed: for b in [past[s] / pool, (past[s] + n_new[s]) / pool), pooled row pool_row0[s] + b <-
+ * mean of the cache rows cache_row0[s] + b * pool .. + pool - 1 (fp32 sum in row order).  max_blocks bounds the blocks of one sequence in this step. */
+int mi355_pool_rows_update(int n_seq, int max_blocks, int width, int pool, const void* cache, int c_dt, int64_t ldc, void* pooled, int p_dt, int64_t ldp,
+                           const int* cache_row0, const int* pool_row0, const int* past, const int* n_new, void* stream);
+/* Rows [n] -> [n].  kind 0 (xIELU; params = fp32 {p, q}): z > 0: softplus(p) z^2 + z / 2; z <= 0: (1/2 + softplus(q)) (exp(z) - 1 - z) + z / 2.
+ * kind 1: out = x * sigmoid(gate), gate rows of dtype g_dt and pitch ldg (params unused). */
+int mi355_act_rows(int64_t rows, int n, const void* x, int x_dt, int64_t ldx, const void* gate, int g_dt, int64_t ldg, int kind, const float* params, void* out,
+                   int out_dt, int64_t ldo, void* stream);
 
 #ifdef __cplusplus
 }

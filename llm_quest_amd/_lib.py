@@ -105,7 +105,7 @@ SIGNATURES = {
     "mi355_embed_hash_fwd": [_L, _I, _I, _P, _P, _P, _F, _P, _I, _I, _I, _P, _P],
     "mi355_add_layernorm_fwd": [_L, _I, _P, _F, _P, _I, _L, _I, _P, _P, _F, _P, _P, _I, _P],
     "mi355_rmsnorm_rows": [_L, _I, _P, _I, _L, _P, _F, _P, _I, _L, _P],
-    "mi355_latent_kv_append": [_L, _I, _I, _P, _I, _L, _P, _F, _P, _P, _P, _I, _P, _I, _L, _P],
+    "mi355_latent_kv_append": [_L, _I, _I, _P, _I, _L, _P, _F, _P, _P, _P, _I, _I, _P, _I, _L, _P],
     "mi355_rope_heads": [_L, _I, _I, _P, _I, _L, _I, _I, _P, _L, _I, _I, _I, _I, _I, _P, _P, _P],
     "mi355_gated_headnorm": [_L, _I, _I, _P, _P, _P, _I, _L, _F, _P, _I, _L, _P],
     "mi355_gla_fwd": [_I, _P, _P, _I, _I, _I, _P, _P, _P, _P, _I, _I, _I, _L, _L, _L, _L, _P, _F, _F, _P, _F, _P, _P, _P],
@@ -113,13 +113,17 @@ SIGNATURES = {
     "mi355_moe_route": [_L, _I, _I, _I, _I, _P, _P, _F, _I, _P, _P, _P],
     "mi355_moe_dispatch": [_L, _I, _P, _P, _P, _P],
     "mi355_bgemm": [_I, _I, _I, _I, _P, _I, _L, _L, _P, _I, _L, _L, _L, _P, _I, _L, _L, _P, _P, _I, _P, _P, _I, _I, _P, _F, _I, _P],
-    "mi355_latent_attn": [_I, _I, _I, _I, _I, _I, _I, _P, _L, _I, _P, _L, _I, _P, _L, _P, _L, _I, _P, _L, _I, _I, _P, _P, _P, _P, _P, _P, _F, _I, _I, _P, _L, _I, _I, _I, _P],
+    "mi355_latent_attn": [_I, _I, _I, _I, _I, _I, _I, _P, _L, _I, _P, _L, _I, _P, _L, _P, _L, _I, _P, _L, _I, _I, _P, _P, _P, _P, _P, _P, _F, _I, _I, _P, _L, _I, _I, _I, _F, _P, _I, _P, _P, _L, _P, _P],
     # parallel-sublayer hybrid decoders in ragged batches (csrc/seqrec.hip)
     "mi355_group_rmsnorm_sum": [_L, _I, _P, _P, _I, _L, _P, _I, _L, _I, _P, _I, _F, _P, _P, _I, _P, _P, _P, _I, _P, _P],
     "mi355_ragged_conv": [_L, _I, _I, _I, _P, _I, _L, _P, _P, _P, _P, _P, _I, _I, _P, _I, _L, _P],
-    "mi355_qkv_rows_append": [_L, _I, _I, _I, _I, _P, _I, _L, _P, _P, _P, _F, _P, _I, _I, _P, _P, _P, _P, _L, _P, _I, _L, _P],
+    "mi355_qkv_rows_append": [_L, _I, _I, _I, _I, _P, _I, _L, _P, _P, _P, _F, _P, _I, _I, _P, _P, _P, _P, _L, _P, _I, _L, _F, _I, _P, _L, _F, _P],
     "mi355_delta_rule_ragged": [_L, _I, _P, _P, _I, _I, _I, _I, _P, _P, _I, _L, _L, _P, _I, _L, _P, _P, _I, _L, _L, _P, _P, _F, _P, _P, _P, _P],
     "mi355_glu_rows": [_L, _I, _P, _I, _L, _I, _F, _P, _I, _L, _P],
+    # decoders with sandwich norms in ragged batches (csrc/seqsand.hip)
+    "mi355_sandwich_rmsnorm": [_L, _I, _P, _P, _I, _L, _P, _P, _P, _F, _P, _I, _P],
+    "mi355_pool_rows_update": [_I, _I, _I, _I, _P, _I, _L, _P, _I, _L, _P, _P, _P, _P, _P],
+    "mi355_act_rows": [_L, _I, _P, _I, _L, _P, _I, _L, _I, _P, _P, _I, _L, _P],
     # measurement aid (csrc/probe.hip)
     "mi355_mfma_pipe_probe": [_I, _I, _P, _P],
     # stand-alone RoPE and dropout (csrc/rope_dropout.hip, csrc/attention_generic.hip)

@@ -8,7 +8,10 @@
 * ``Retention``             -- linear attention with one fixed decay per head (rotate-half rotary, gated unit-RMS output);
 * ``SlidingWindowAttention``-- grouped-query softmax attention with biases, query / key norm, a temperature per head and a window that keeps the first tokens;
 * ``GatedDeltaRule``        -- the gated delta rule behind short convolutions, unit-vector queries and keys, a matrix state per value head in fp32;
-* ``GatedMLP`` / ``SoftmaxTopkMoE`` -- a dense GELU-gated layer; softmax-routed experts with a clamped gated activation, weights = the winners' scores.
+* ``GatedMLP`` / ``SoftmaxTopkMoE`` -- a dense GELU-gated layer; softmax-routed experts with a clamped gated activation, weights = the winners' scores;
+* ``ActMLP``                -- an un-gated feed-forward around the xIELU activation.
+``LatentAttention`` also runs without a query latent, with rotate-half rotary, a sliding window and a sigmoid output gate; ``SlidingWindowAttention`` also
+with capped scores, a position-dependent query temperature, pooled blocks before the window, a sink in the denominator and value mixing between layers.
 
 They run one *step* of a batch (``SeqStep``): the new tokens of every sequence, packed row after row, against what ``utils.SlotStateCache`` holds.  Inference
 only, HIP kernels only (``kernels_seq``); weights are bf16, what is normalised, rotated, decayed, accumulated over time or routed is fp32.
@@ -44,7 +47,7 @@ class SeqStep:
         self.T, self.n_seq, self.max_new = seq_off[-1], len(slots), max(n_new)
         self.max_keys = max(p + n for p, n in zip(past, n_new))
         self.fresh = all(p == 0 for p in past)
-        self.host_seq_off = seq_off
+        self.host_seq_off, self.host_past, self.host_n_new = seq_off, past, n_new
         T, n = self.T, self.n_seq
         row0 = [s * cap for s in slots]
         # rows of the descriptor block: tokens | previous token | position | cache row | per-sequence arrays | 0 .. T-1 | sequence of a row; one
@@ -73,6 +76,18 @@ class SeqStep:
         (self.tok, self.prev, self.pos, self.dst_row, self.seq_off, self.slots, self.past, self.n_new, self.cache_row0, self.local_row, self.row_seq) = parts
         self.q_row0 = self.seq_off[:n]
         self.local = {}  # layer -> this step's latent rows [T, rank + rot] (prompts: the expanded form reads them instead of the cache)
+        self.shared = {}  # what one layer leaves for later layers of the same step (the first value-mixing layer's values)
+        self._pool_row0 = {}
+
+    def pool_row0(self, blocks_per_slot):
+        """int32 [n_seq]: the first pooled row of every sequence in a buffer with ``blocks_per_slot`` rows per slot."""
+        if blocks_per_slot not in self._pool_row0:
+            self._pool_row0[blocks_per_slot] = (self.slots * blocks_per_slot).to(I32).contiguous()
+        return self._pool_row0[blocks_per_slot]
+
+    def completed_blocks(self, pool):
+        """The most blocks of ``pool`` positions that one sequence of the step completes."""
+        return max((p + n) // pool - p // pool for p, n in zip(self.host_past, self.host_n_new))
 
 
 def _f32(t):
@@ -88,20 +103,27 @@ class _Frozen(nn.Module):
 
 class LatentAttention(_Frozen):
     """Multi-head latent attention.  Per head ``dim`` unrotated + ``rot_dim`` rotated query / key entries, ``vdim`` values; latents of ``q_rank`` /
-    ``kv_rank``.  ``kv_from``: read that layer's cached rows instead of projecting own ones.  Rotary: interleaved pairs, ``rot_dims`` of the rotated part
-    turn (base ``rot_base``)."""
+    ``kv_rank``.  ``kv_from``: read that layer's cached rows instead of projecting own ones.  Rotary: ``rot_dims`` of the rotated part turn (base
+    ``rot_base``), as interleaved pairs or -- ``rot_layout`` 1 -- entry i with entry i + rot_dims / 2.  ``q_rank`` 0: the query is projected from the
+    input directly, without a latent.  ``window`` > 0: position i sees the keys j with 0 <= i - j < window.  ``gate``: the concatenated heads are multiplied
+    by the sigmoid of a projection of the mixer's input before the output projection."""
 
-    def __init__(self, width, heads, dim, rot_dim, vdim, q_rank, kv_rank, scale, rot_dims, rot_base, eps, layer_idx, kv_from=None):
+    def __init__(self, width, heads, dim, rot_dim, vdim, q_rank, kv_rank, scale, rot_dims, rot_base, eps, layer_idx, kv_from=None, rot_layout=0, window=0, gate=False):
         super().__init__()
         self.width, self.heads, self.dim, self.rot_dim, self.vdim = width, heads, dim, rot_dim, vdim
         self.q_rank, self.kv_rank, self.scale, self.rot_dims, self.rot_base, self.eps = q_rank, kv_rank, float(scale), rot_dims, float(rot_base), float(eps)
         self.layer_idx, self.kv_from = layer_idx, kv_from
+        self.rot_layout, self.window, self.gate = int(rot_layout), int(window), bool(gate)
+        if rot_dims % 2 or rot_dims > rot_dim:
+            raise ValueError("LatentAttention: the rotated entries are an even number <= rot_dim")
         own = kv_from is None
-        # down projections side by side: [q_rank | kv_rank + rot_dim] rows -> one product
-        self.w_down = self._param(q_rank + (kv_rank + rot_dim if own else 0), width)
-        self.q_norm = self._param(q_rank)
+        # projections of the input side by side -> one product: [query latent, or the queries themselves | kv_rank + rot_dim | gate]
+        self.q_cols = q_rank if q_rank else heads * (dim + rot_dim)
+        self.kv_cols = kv_rank + rot_dim if own else 0
+        self.w_down = self._param(self.q_cols + self.kv_cols + (heads * vdim if gate else 0), width)
+        self.q_norm = self._param(q_rank) if q_rank else None
         self.kv_norm = self._param(kv_rank) if own else None
-        self.w_uq = self._param(heads * (dim + rot_dim), q_rank)
+        self.w_uq = self._param(heads * (dim + rot_dim), q_rank) if q_rank else None
         self.w_ukv = self._param(heads * (dim + vdim), kv_rank)  # [key up-projection | value up-projection] rows
         self.w_o = self._param(width, heads * vdim)
         self._ready = None
@@ -117,46 +139,51 @@ class LatentAttention(_Frozen):
             self._ready = device
 
     @torch.no_grad()
-    def step(self, h, st):
-        """h [T, width] in the activation dtype -> the mixer's output rows [T, width]."""
+    def step(self, h, st, out_dtype=None):
+        """h [T, width] in the activation dtype -> the mixer's output rows [T, width] (``out_dtype``: of the output projection; default h's)."""
         self.prepare(h.device)
-        H, dn, dr, dv, R, Rq = self.heads, self.dim, self.rot_dim, self.vdim, self.kv_rank, self.q_rank
+        H, dn, dr, dv, R, Rq = self.heads, self.dim, self.rot_dim, self.vdim, self.kv_rank, self.q_cols
         own = self.kv_from is None
         src = self.layer_idx if own else self.kv_from
         cache2d = st.cache.rows2d(self.layer_idx)
-        down = S.linear(h, self.w_down)
-        q = S.linear(S.rmsnorm_rows(down[:, :Rq], self.q_norm32, self.eps), self.w_uq)
+        lay, win = self.rot_layout, self.window
+        # without a query latent the projection feeds fp32 work only (rotary, the latent's norm, the gate's sigmoid): it leaves the product as fp32
+        down = S.linear(h, self.w_down, out_dtype=None if self.q_rank else F32)
+        q = S.linear(S.rmsnorm_rows(down[:, :Rq], self.q_norm32, self.eps), self.w_uq) if self.q_rank else down[:, :Rq]
+        kv_src = down[:, Rq : Rq + self.kv_cols]
         if own:
-            S.latent_kv_append(down[:, Rq:], R, dr, self.kv_norm32, self.eps, st.pos, st.dst_row, self.freq, self.rot_dims, cache2d)
+            S.latent_kv_append(kv_src, R, dr, self.kv_norm32, self.eps, st.pos, st.dst_row, self.freq, self.rot_dims, cache2d, layout=lay)
         T = h.shape[0]
         if st.fresh:
             # prompts: keys and values per head rebuilt from this step's latent rows, ordinary head-by-head attention
             if own:
                 lat = torch.empty((T, R + dr), dtype=st.act_dtype, device=h.device)
-                S.latent_kv_append(down[:, Rq:], R, dr, self.kv_norm32, self.eps, st.pos, st.local_row, self.freq, self.rot_dims, lat)
+                S.latent_kv_append(kv_src, R, dr, self.kv_norm32, self.eps, st.pos, st.local_row, self.freq, self.rot_dims, lat, layout=lay)
                 st.local[src] = lat
             lat = st.local[src]
             kv = S.linear(lat[:, :R], self.w_ukv)  # [T, H*dn | H*dv]
             q32 = torch.empty((T, H * (dn + dr)), dtype=F32, device=h.device)
-            S.rope_heads(q, H, dn + dr, dn + dr, 0, q32, dn + dr, 0, dn, self.rot_dims, self.freq, st.pos)
+            S.rope_heads(q, H, dn + dr, dn + dr, 0, q32, dn + dr, 0, dn, self.rot_dims, self.freq, st.pos, layout=lay)
             ctx = torch.empty((T, H * dv), dtype=st.act_dtype, device=h.device)
             S.latent_attn(q32, kv[:, : H * dn], lat[:, R:], kv[:, H * dn :], ctx, H, 1, dn, dr, dv, dn + dr, dn, dv, dv,
-                          (st.q_row0, st.n_new, st.past, st.q_row0, st.q_row0, st.q_row0), st.max_new, self.scale)
+                          (st.q_row0, st.n_new, st.past, st.q_row0, st.q_row0, st.q_row0), st.max_new, self.scale, window=win)
         else:
             # continuation: the key up-projection folded onto the query, the value up-projection applied after the attention -- the cache rows are
             # keys and values of every head as they stand
             qf = torch.empty((T, H * (R + dr)), dtype=F32, device=h.device)
             S.bgemm(q, self.w_ukv, qf, T, R, dn, batch=H, lda=q.stride(0), a_bs=dn + dr, sbn=1, sbk=R, b_bs=dn * R, ldc=H * (R + dr), c_bs=R + dr)
-            S.rope_heads(q, H, dr, dn + dr, dn, qf, R + dr, R, 0, self.rot_dims, self.freq, st.pos)
+            S.rope_heads(q, H, dr, dn + dr, dn, qf, R + dr, R, 0, self.rot_dims, self.freq, st.pos, layout=lay)
             hm = 1
             while hm < min(H, 32):
                 hm *= 2
             ol = torch.empty((T, H * R), dtype=st.act_dtype, device=h.device)
             S.latent_attn(qf, cache2d, cache2d[:, R:], cache2d, ol, H, hm, R, dr, R, R + dr, 0, 0, R,
-                          (st.q_row0, st.n_new, st.past, st.cache_row0, st.cache_row0, st.cache_row0), st.max_new, self.scale, max_keys=st.max_keys)
+                          (st.q_row0, st.n_new, st.past, st.cache_row0, st.cache_row0, st.cache_row0), st.max_new, self.scale, max_keys=st.max_keys, window=win)
             ctx = torch.empty((T, H * dv), dtype=st.act_dtype, device=h.device)
             S.bgemm(ol, self.w_ukv[H * dn :], ctx, T, dv, R, batch=H, lda=H * R, a_bs=R, sbn=R, sbk=1, b_bs=dv * R, ldc=H * dv, c_bs=dv)
-        return S.linear(ctx, self.w_o)
+        if self.gate:
+            ctx = S.act_rows(ctx, S.ACT_SIGMOID_GATE, gate=down[:, Rq + self.kv_cols :])
+        return S.linear(ctx, self.w_o, out_dtype=out_dtype)
 
 
 class GatedLinearAttention(_Frozen):
@@ -304,52 +331,89 @@ class Retention(_Frozen):
 
 
 class SlidingWindowAttention(_Frozen):
-    """Grouped-query softmax attention with biases on the four projections, an RMS norm (one weight for all heads) on every query and key head before
-    an interleaved rotary embedding of the first ``rot_dims`` entries, score = q.k * scale * temp[h], and a causal sliding window that also keeps the
+    """Grouped-query softmax attention with optional biases on the four projections, an optional RMS norm (one weight for all heads) on every query and key
+    head before a rotary embedding of the first ``rot_dims`` entries, score = q.k * scale * temp[h], and a causal sliding window that also keeps the
     first tokens: position i sees j <= i if i - j < window or j < keep_first (window 0: all of them).  Keys and values are cached token-major,
-    [kv_heads x dim | kv_heads x vdim] per row."""
+    [kv_heads x dim | kv_heads x vdim] per row.  Further options, each a constant of its own:
+      * ``softcap`` > 0      -- the scaled score passes softcap * tanh(score / softcap);
+      * ``q_temp`` (coef, every) -- the query at position p is multiplied by 1 + coef * ln(floor((p + 1) / every) + 1);
+      * ``pool`` > 0         -- besides the window, one key and one value for every block of ``pool`` tokens that lies wholly before the window, block b
+        being seen from position i iff (b + 1) pool - 1 <= i - window; they are the means of the block's cached keys / values and share the softmax;
+      * ``sink``             -- a learned number per head whose exponential joins the softmax denominator (no key, no value, not scaled);
+      * ``v_mix`` ("first" / "mix") -- the first such layer of a step leaves its values for the later ones, which cache (1 - lam) v + lam v_first."""
 
-    def __init__(self, width, heads, kv_heads, dim, vdim, scale, window, keep_first, rot_dims, rot_base, eps, layer_idx, qk_norm=True, bias=True, temp=True):
+    def __init__(self, width, heads, kv_heads, dim, vdim, scale, window, keep_first, rot_dims, rot_base, eps, layer_idx, qk_norm=True, bias=True, temp=True,
+                 softcap=0.0, q_temp=None, pool=0, sink=False, v_mix=None):
         super().__init__()
         if heads % kv_heads:
             raise ValueError("SlidingWindowAttention: heads must be a multiple of kv_heads")
         if rot_dims % 2 or rot_dims > dim:
             raise ValueError("SlidingWindowAttention: the rotated entries are an even number <= dim")
+        if pool and (not window or keep_first):
+            raise ValueError("SlidingWindowAttention: pooled blocks lie before a window (and exclude kept first tokens)")
+        if v_mix not in (None, "first", "mix"):
+            raise ValueError("SlidingWindowAttention: v_mix is None, 'first' or 'mix'")
         self.width, self.heads, self.kv_heads, self.dim, self.vdim, self.scale, self.window, self.keep_first = width, heads, kv_heads, dim, vdim, float(scale), int(window), int(keep_first)
         self.rot_dims, self.rot_base, self.eps, self.layer_idx = rot_dims, float(rot_base), float(eps), layer_idx
+        self.softcap, self.q_temp, self.pool, self.v_mix = float(softcap or 0.0), (float(q_temp[0]), int(q_temp[1])) if q_temp else None, int(pool or 0), v_mix
         n = (heads + kv_heads) * dim + kv_heads * vdim
         self.w_qkv = self._param(n, width)
         self.b_qkv = self._param(n) if bias else None
         self.q_norm = self._param(dim) if qk_norm else None
         self.k_norm = self._param(dim) if qk_norm else None
         self.temp = self._param(heads) if temp else None
+        self.sink = self._param(heads) if sink else None
+        self.lam = self._param(1) if v_mix == "mix" else None
         self.w_o = self._param(width, heads * vdim)
         self.b_o = self._param(width) if bias else None
         self._ready = None
 
     def cache_spec(self):
-        return {"rows": self.kv_heads * (self.dim + self.vdim), "states": {}}
+        spec = {"rows": self.kv_heads * (self.dim + self.vdim), "states": {}}
+        if self.pool:
+            spec["pool"] = self.pool
+        return spec
 
     def prepare(self, device):
         if self._ready != device:
-            self.b_qkv32, self.q_norm32, self.k_norm32, self.b_o32 = _f32(self.b_qkv), _f32(self.q_norm), _f32(self.k_norm), _f32(self.b_o)
+            self.b_qkv32, self.q_norm32, self.k_norm32, self.b_o32, self.sink32 = _f32(self.b_qkv), _f32(self.q_norm), _f32(self.k_norm), _f32(self.b_o), _f32(self.sink)
             t = _f32(self.temp) if self.temp is not None else torch.ones(self.heads, dtype=F32, device=device)
-            self.qscale = (t * self.scale).contiguous()  # the score's two factors, folded onto the query
+            # the score's factors: folded onto the query, unless the scaled score goes through the cap (then the kernel scales)
+            self.qscale = None if self.softcap else (t * self.scale).contiguous()
+            if self.softcap and self.temp is not None:
+                raise ValueError("SlidingWindowAttention: a per-head temperature and a score cap do not combine")
             self.freq = S.rope_frequencies(self.rot_dims, self.rot_base, device) if self.rot_dims else None
+            self.lam32 = float(self.lam.float().item()) if self.lam is not None else 0.0
             self._ready = device
 
     @torch.no_grad()
-    def step(self, h, st):
+    def step(self, h, st, out_dtype=None):
         self.prepare(h.device)
         H, G, d, dv = self.heads, self.kv_heads, self.dim, self.vdim
-        cache2d = st.cache.rows2d(self.layer_idx)
+        L_ = self.layer_idx
+        cache2d = st.cache.rows2d(L_)
         proj = S.linear(h, self.w_qkv, out_dtype=F32)
-        q = S.qkv_rows_append(proj, H, G, d, dv, self.b_qkv32, self.q_norm32, self.k_norm32, self.eps, self.qscale, self.rot_dims, 0, self.freq, st.pos, st.dst_row, cache2d)
+        vmix = None
+        if self.v_mix == "mix":
+            vmix = st.shared["v_first"]
+            if vmix.shape[1] != G * dv:
+                raise ValueError("SlidingWindowAttention: value-mixing layers share one value width")
+        elif self.v_mix == "first":
+            st.shared["v_first"] = proj[:, (H + G) * d :]  # this step's unmixed values (a view: proj stays alive with it)
+        q = S.qkv_rows_append(proj, H, G, d, dv, self.b_qkv32, self.q_norm32, self.k_norm32, self.eps, self.qscale, self.rot_dims, 0, self.freq, st.pos, st.dst_row, cache2d,
+                              q_temp=self.q_temp, vmix=vmix, lam=self.lam32)
+        pooled = row0 = None
+        if self.pool:
+            p2d = st.cache.pooled2d(L_)
+            row0 = st.pool_row0(st.cache.pool_capacity(L_))
+            S.pool_rows_update(cache2d, p2d, self.pool, st.cache_row0, row0, st.past, st.n_new, st.completed_blocks(self.pool))
+            pooled = (p2d, p2d[:, G * d :])
         ctx = torch.empty((h.shape[0], H * dv), dtype=st.act_dtype, device=h.device)
         hm = _largest_pow2_divisor(H // G)
         S.latent_attn(q, cache2d, None, cache2d[:, G * d :], ctx, H, hm, d, 0, dv, d, d, dv, dv, (st.q_row0, st.n_new, st.past, st.cache_row0, st.cache_row0, st.cache_row0),
-                      st.max_new, 1.0, max_keys=st.max_keys, kv_rep=H // G, window=self.window, keep_first=self.keep_first)
-        return S.linear(ctx, self.w_o, bias=self.b_o32)
+                      st.max_new, self.scale if self.softcap else 1.0, max_keys=st.max_keys, kv_rep=H // G, window=self.window, keep_first=self.keep_first,
+                      softcap=self.softcap, sink=self.sink32, pool=self.pool, pooled=pooled, pool_row0=row0)
+        return S.linear(ctx, self.w_o, bias=self.b_o32, out_dtype=out_dtype)
 
 
 class GatedDeltaRule(_Frozen):
@@ -443,3 +507,26 @@ class SoftmaxTopkMoE(_Frozen):
         out = torch.empty((T * top, self.width), dtype=F32, device=h.device)
         S.bgemm(act, self.w_down, out, T * top, self.width, ff, batch=E, sbn=ff, b_bs=self.width * ff, grp_offs=offs, c_rows=perm, row_scale=wts.view(-1))
         return out
+
+
+class ActMLP(_Frozen):
+    """Un-gated feed-forward: down(act(up x)) with the xIELU activation -- z > 0: softplus(p) z^2 + z / 2; z <= 0: (1/2 + softplus(q)) (exp(z) - 1 - z) + z / 2,
+    p and q two learned numbers of the layer."""
+
+    def __init__(self, width, ff):
+        super().__init__()
+        self.width, self.ff = width, ff
+        self.w_up = self._param(ff, width)
+        self.w_down = self._param(width, ff)
+        self.act = self._param(2)
+        self._ready = None
+
+    def prepare(self, device):
+        if self._ready != device:
+            self.act32 = _f32(self.act)
+            self._ready = device
+
+    @torch.no_grad()
+    def step(self, h, out_dtype=None):
+        self.prepare(h.device)
+        return S.linear(S.act_rows(S.linear(h, self.w_up), S.ACT_XIELU, params=self.act32), self.w_down, out_dtype=out_dtype)

@@ -6,7 +6,10 @@
 //
 // score(row, j) = scale * ( Q[row, :D1] . K1[j, head, :] + Q[row, D1:] . K2[j, :] ),  softmax over j <= past + token index, out = sum_j p V[j].
 // The same kernels serve grouped-query attention (kv_rep query heads per key / value head, D2 = 0) and a sliding window that keeps the first tokens
-// (window, keep_first): key steps that no row of a tile can see are skipped.
+// (window, keep_first): key steps that no row of a tile can see are skipped.  Further options: tanh-capped scores (softcap), a per-head sink that
+// only enters the softmax denominator, and POOLED blocks in front of a window -- one mean key / value row per `pool` tokens, kept by the caller in a
+// second buffer; the query at position i sees block b iff all of its tokens have left the window, (b + 1) pool <= i - window + 1.  Pooled rows
+// and tokens share one softmax: the key loop simply runs over the pooled rows first.
 // Scores, softmax statistics and the output accumulators are fp32.  A tile is `tm` tokens x `hm` heads = 32 query rows (hm > 1 only with shared
 // keys and values) against 64 keys at a time.
 //
@@ -31,7 +34,21 @@ struct LatAttnArgs {
     int kv_rep;  // query heads per key / value head (grouped queries): head h reads key / value head h / kv_rep
     int window;  // > 0: a query at position i sees key j <= i only if i - j < window or j < keep_first (sliding window that keeps the first tokens)
     int keep_first;
+    float softcap;      // > 0: score <- softcap * tanh(score / softcap) after the scale
+    const float* sink;  // fp32 [H] or NULL: exp(sink[h]) joins the denominator of head h (no key, no value, not scaled)
+    int pool;           // > 0: one pooled key / value row per `pool` tokens (needs window > 0, D2 == 0); rows PK / PV, first row of sequence s = pool_row0[s]
+    const void *PK, *PV;
+    int64_t ldp;
+    const int* pool_row0;
 };
+
+// pooled blocks the query at position lim sees: those that end at or before lim - window
+__device__ __forceinline__ int pooled_visible(int lim, int window, int pool) {
+    const int gone = lim - window + 1;  // tokens that have left the window
+    return gone > 0 ? gone / pool : 0;
+}
+// the capped score (natural units)
+__device__ __forceinline__ float cap_score(float s, float cap) { return cap > 0.f ? cap * tanhf(s / cap) : s; }
 
 // key j for the query at position lim (lim < 0: a padding row that sees nothing)
 __device__ __forceinline__ bool key_visible(int j, int lim, int window, int keep_first) { return j <= lim && (window <= 0 || lim - j < window || j < keep_first); }
@@ -74,8 +91,23 @@ __global__ __launch_bounds__(256) void latent_attn_fma_kernel(LatAttnArgs p) {
 
     const int kvh = head0 / p.kv_rep;
     const int win_lo = p.window > 0 ? past + tok0 - p.window + 1 : 0;  // keys below it are outside the window of every row of the tile
-    for (int j0 = 0; j0 < n_keys; j0 += AN) {
-        if (j0 + AN <= win_lo && j0 >= p.keep_first) continue;  // block-uniform: no row sees a key of this step
+    const int n_pool = p.pool > 0 ? pooled_visible(n_keys - 1, p.window, p.pool) : 0;  // pooled rows any row of the tile may see
+    const int pool_steps = (n_pool + AN - 1) / AN;
+    const int64_t pr0 = p.pool > 0 ? p.pool_row0[s] : 0;
+    int npv[2];
+#pragma unroll
+    for (int a = 0; a < 2; ++a) npv[a] = p.pool > 0 ? pooled_visible(lim[a], p.window, p.pool) : 0;
+    for (int it = -pool_steps;; ++it) {
+        const bool seg = it < 0;  // the pooled rows come first
+        const int j0 = seg ? (it + pool_steps) * AN : it * AN;
+        const int n_here = seg ? n_pool : n_keys;
+        if (!seg) {
+            if (j0 >= n_keys) break;
+            if (j0 + AN <= win_lo && j0 >= p.keep_first) continue;  // block-uniform: no row sees a key of this step
+        }
+        const void* Kp = seg ? p.PK : p.K1;
+        const void* Vp = seg ? p.PV : p.V;
+        const int64_t kr = seg ? pr0 : k1r0, vr = seg ? pr0 : vr0, ldk = seg ? p.ldp : p.ldk1, ldvv = seg ? p.ldp : p.ldv;
         float acc[2][4] = {};
         for (int d0 = 0; d0 < DK; d0 += AC) {
             __syncthreads();
@@ -89,8 +121,8 @@ __global__ __launch_bounds__(256) void latent_attn_fma_kernel(LatAttnArgs p) {
             for (int i = 0; i < 8; ++i) {  // K chunk: 64 keys x 32 features
                 const int e = tid + 256 * i, d = d0 + (e & 31), j = j0 + (e >> 5);
                 float v = 0.f;
-                if (j < n_keys && d < DK)
-                    v = d < p.D1 ? lda_dt(p.K1, p.dt, (k1r0 + j) * p.ldk1 + (int64_t)kvh * p.k1_hs + d) : lda_dt(p.K2, p.dt, (k2r0 + j) * p.ldk2 + (d - p.D1));
+                if (j < n_here && d < DK)
+                    v = d < p.D1 ? lda_dt(Kp, p.dt, (kr + j) * ldk + (int64_t)kvh * p.k1_hs + d) : lda_dt(p.K2, p.dt, (k2r0 + j) * p.ldk2 + (d - p.D1));
                 Ks[e >> 5][e & 31] = v;
             }
             __syncthreads();
@@ -112,7 +144,8 @@ __global__ __launch_bounds__(256) void latent_attn_fma_kernel(LatAttnArgs p) {
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 const int j = j0 + tx + 16 * i;
-                acc[a][i] = key_visible(j, lim[a], p.window, p.keep_first) ? acc[a][i] * p.scale : -__builtin_huge_valf();
+                const bool vis = seg ? j < npv[a] : key_visible(j, lim[a], p.window, p.keep_first);
+                acc[a][i] = vis ? cap_score(acc[a][i] * p.scale, p.softcap) : -__builtin_huge_valf();
                 mx = fmaxf(mx, acc[a][i]);
             }
 #pragma unroll
@@ -135,7 +168,7 @@ __global__ __launch_bounds__(256) void latent_attn_fma_kernel(LatAttnArgs p) {
         }
         __syncthreads();
         // O <- O * f + P V
-        const int nk = min(AN, n_keys - j0);
+        const int nk = min(AN, n_here - j0);
 #pragma unroll
         for (int r = 0; r < 8; ++r) {
             const float f = fs[8 * rg + r];
@@ -147,7 +180,7 @@ __global__ __launch_bounds__(256) void latent_attn_fma_kernel(LatAttnArgs p) {
 #pragma unroll
             for (int i = 0; i < NC; ++i) {
                 const int col = c + 64 * i;
-                vv[i] = col < p.DV ? lda_dt(p.V, p.dt, (vr0 + j0 + j) * p.ldv + (int64_t)kvh * p.v_hs + col) : 0.f;
+                vv[i] = col < p.DV ? lda_dt(Vp, p.dt, (vr + j0 + j) * ldvv + (int64_t)kvh * p.v_hs + col) : 0.f;
             }
 #pragma unroll
             for (int r = 0; r < 8; ++r) {
@@ -158,13 +191,25 @@ __global__ __launch_bounds__(256) void latent_attn_fma_kernel(LatAttnArgs p) {
         }
     }
     __syncthreads();
-    if (tx == 0) ls[2 * ty] = l_run[0], ls[2 * ty + 1] = l_run[1];
+    if (tx == 0) {
+#pragma unroll
+        for (int a = 0; a < 2; ++a) {
+            const int r = 2 * ty + a, head = head0 + r % p.hm;
+            float l = l_run[a], f = 1.0f;
+            if (p.sink && head < p.H) {  // the sink joins the denominator: out = O f / (l f + exp(sink - m'))
+                const float sk = p.sink[head], m2 = fmaxf(m_run[a], sk);
+                f = expf(m_run[a] - m2);
+                l = l * f + expf(sk - m2);
+            }
+            ls[r] = l, fs[r] = f;
+        }
+    }
     __syncthreads();
 #pragma unroll
     for (int r = 0; r < 8; ++r) {
         const int row = 8 * rg + r, tok = tok0 + row / p.hm, head = head0 + row % p.hm;
         if (tok >= n_new || head >= p.H) continue;
-        const float inv = 1.0f / ls[row];
+        const float inv = fs[row] / ls[row];
         const int64_t ob = (qr0 + tok) * p.ldo + (int64_t)head * p.o_hs;
 #pragma unroll
         for (int i = 0; i < NC; ++i) {
@@ -243,16 +288,31 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(LatAttnArgs p, in
 
     const int kvh = head0 / p.kv_rep;
     const int win_lo = p.window > 0 ? past + tok0 - p.window + 1 : 0;
-    for (int j0 = key_lo; j0 < n_keys; j0 += MKT) {
-        if (j0 + MKT <= win_lo && j0 >= p.keep_first) continue;  // block-uniform: no row sees a key of this step
+    // pooled rows any row of the tile may see (a tile's first key share takes them), and those this lane's query sees
+    const int n_pool = (p.pool > 0 && split == 0) ? pooled_visible(past + min(tok0 + tm, n_new) - 1, p.window, p.pool) : 0;
+    const int pool_steps = (n_pool + MKT - 1) / MKT;
+    const int npv = p.pool > 0 ? pooled_visible(lim, p.window, p.pool) : 0;
+    const int64_t pr0 = p.pool > 0 ? p.pool_row0[s] : 0;
+    const float capl = p.softcap * 1.4426950408889634f;
+    for (int it = -pool_steps;; ++it) {
+        const bool seg = it < 0;  // the pooled rows come first
+        const int j0 = seg ? (it + pool_steps) * MKT : key_lo + it * MKT;
+        const int n_here = seg ? n_pool : n_keys;
+        if (!seg) {
+            if (j0 >= n_keys) break;
+            if (j0 + MKT <= win_lo && j0 >= p.keep_first) continue;  // block-uniform: no row sees a key of this step
+        }
+        const bf16_t* Kp = seg ? (const bf16_t*)p.PK : K1;
+        const bf16_t* Vp = seg ? (const bf16_t*)p.PV : V;
+        const int64_t kr = seg ? pr0 : k1r0, vr = seg ? pr0 : vr0, ldk = seg ? p.ldp : p.ldk1, ldvv = seg ? p.ldp : p.ldv;
         __syncthreads();
         // ---- key tile -> LDS
         for (int c = tid; c < MKT * DKS; c += 256) {
             const int key = c / DKS, d0 = (c % DKS) * 8, j = j0 + key;
             u32x4 val = {0u, 0u, 0u, 0u};
-            if (j < n_keys) {
+            if (j < n_here) {
                 if (vec_ok && d0 + 8 <= p.D1) {
-                    val = *(const u32x4*)(K1 + (k1r0 + j) * p.ldk1 + (int64_t)kvh * p.k1_hs + d0);
+                    val = *(const u32x4*)(Kp + (kr + j) * ldk + (int64_t)kvh * p.k1_hs + d0);
                 } else if (vec_ok && d0 >= p.D1 && d0 + 8 <= DK) {
                     val = *(const u32x4*)(K2 + (k2r0 + j) * p.ldk2 + (d0 - p.D1));
                 } else {
@@ -260,7 +320,7 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(LatAttnArgs p, in
 #pragma unroll
                     for (int i = 0; i < 8; ++i) {
                         const int d = d0 + i;
-                        e[i] = d < p.D1 ? K1[(k1r0 + j) * p.ldk1 + (int64_t)kvh * p.k1_hs + d] : (d < DK ? K2[(k2r0 + j) * p.ldk2 + (d - p.D1)] : (bf16_t)0);
+                        e[i] = d < p.D1 ? Kp[(kr + j) * ldk + (int64_t)kvh * p.k1_hs + d] : (d < DK ? K2[(k2r0 + j) * p.ldk2 + (d - p.D1)] : (bf16_t)0);
                     }
                     val = u32x4{(unsigned)e[0] | ((unsigned)e[1] << 16), (unsigned)e[2] | ((unsigned)e[3] << 16), (unsigned)e[4] | ((unsigned)e[5] << 16),
                                 (unsigned)e[6] | ((unsigned)e[7] << 16)};
@@ -274,19 +334,19 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(LatAttnArgs p, in
         for (int c = tid; c < MKT * (DVP / 8); c += 256) {
             const int key = c % MKT, v0 = (c / MKT) * 8, j = j0 + key;
             bf16_t e[8];
-            if (j < n_keys && vec_ok && v0 + 8 <= p.DV) {
-                const u32x4 val = *(const u32x4*)(V + (vr0 + j) * p.ldv + (int64_t)kvh * p.v_hs + v0);
+            if (j < n_here && vec_ok && v0 + 8 <= p.DV) {
+                const u32x4 val = *(const u32x4*)(Vp + (vr + j) * ldvv + (int64_t)kvh * p.v_hs + v0);
 #pragma unroll
                 for (int i = 0; i < 4; ++i) e[2 * i] = (bf16_t)(val[i] & 0xffffu), e[2 * i + 1] = (bf16_t)(val[i] >> 16);
             } else {
 #pragma unroll
-                for (int i = 0; i < 8; ++i) e[i] = (j < n_keys && v0 + i < p.DV) ? V[(vr0 + j) * p.ldv + (int64_t)kvh * p.v_hs + v0 + i] : (bf16_t)0;
+                for (int i = 0; i < 8; ++i) e[i] = (j < n_here && v0 + i < p.DV) ? Vp[(vr + j) * ldvv + (int64_t)kvh * p.v_hs + v0 + i] : (bf16_t)0;
             }
 #pragma unroll
             for (int i = 0; i < 8; ++i) Vt[(v0 + i) * VLD + key] = e[i];
         }
         __syncthreads();
-        if (j0 > wave_lim) continue;  // every key of this step lies behind the wave's rows (the barriers above are still reached by all)
+        if (!seg && j0 > wave_lim) continue;  // every key of this step lies behind the wave's rows (the barriers above are still reached by all)
         // ---- S^T = K Q^T: two blocks of 32 keys
         f32x16 sacc[2];
 #pragma unroll
@@ -306,7 +366,8 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(LatAttnArgs p, in
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
                 const int j = j0 + kb * 32 + 8 * (r >> 2) + 4 * hf + (r & 3);
-                const float v = (key_visible(j, lim, p.window, p.keep_first) && j < n_keys) ? sacc[kb][r] * sc2 : NEG;
+                const bool vis = seg ? j < npv : (key_visible(j, lim, p.window, p.keep_first) && j < n_keys);
+                const float v = !vis ? NEG : (p.softcap > 0.f ? capl * tanhf(sacc[kb][r] * p.scale / p.softcap) : sacc[kb][r] * sc2);
                 sacc[kb][r] = v;
                 mx = fmaxf(mx, v);
             }
@@ -355,7 +416,11 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(LatAttnArgs p, in
         return;
     }
     if (!row_ok) return;
-    const float inv = 1.0f / l_run;
+    float inv = 1.0f / l_run;
+    if (p.sink) {  // the sink joins the denominator (statistics are in base-2 units)
+        const float sk = p.sink[head] * 1.4426950408889634f, m2 = fmaxf(m_run, sk), f = exp2f(m_run - m2);
+        inv = f / (l_run * f + exp2f(sk - m2));
+    }
     bf16_t* orow = (bf16_t*)p.O + (qr0 + tok) * p.ldo + (int64_t)head * p.o_hs;
 #pragma unroll
     for (int vb = 0; vb < NVB; ++vb)
@@ -383,6 +448,11 @@ __global__ __launch_bounds__(256) void latent_attn_combine_kernel(LatAttnArgs p,
     float m = -__builtin_huge_valf();
     for (int i = 0; i < p.splits; ++i) m = fmaxf(m, p.ws[(blk0 + i) * stride + row]);
     float l = 0.f;
+    if (p.sink) {
+        const float sk = p.sink[head] * 1.4426950408889634f;
+        m = fmaxf(m, sk);
+        l = exp2f(sk - m);
+    }
     for (int i = 0; i < p.splits; ++i) {
         const float mi = p.ws[(blk0 + i) * stride + row];
         if (mi != -__builtin_huge_valf()) l += p.ws[(blk0 + i) * stride + MQ + row] * exp2f(mi - m);
@@ -410,7 +480,8 @@ static int launch_mfma(const LatAttnArgs& p, dim3 grid, int vec_ok, hipStream_t 
 extern "C" int mi355_latent_attn(int n_seq, int max_new, int H, int hm, int D1, int D2, int DV, const float* Q, int64_t ldq, int q_hs, const void* K1, int64_t ldk1,
                                  int k1_hs, const void* K2, int64_t ldk2, const void* V, int64_t ldv, int v_hs, void* O, int64_t ldo, int o_hs, int dt,
                                  const int* q_row0, const int* n_new, const int* past, const int* k1_row0, const int* k2_row0, const int* v_row0, float scale,
-                                 int use_mfma, int splits, float* ws, int64_t ws_floats, int kv_rep, int window, int keep_first, void* stream) {
+                                 int use_mfma, int splits, float* ws, int64_t ws_floats, int kv_rep, int window, int keep_first, float softcap, const float* sink,
+                                 int pool, const void* PK, const void* PV, int64_t ldp, const int* pool_row0, void* stream) {
     MI355_REQUIRE(n_seq > 0 && n_seq <= 65535 && max_new > 0 && H > 0 && D1 > 0 && D2 >= 0 && DV > 0 && DV <= 512 && Q && K1 && V && O && (D2 == 0 || K2),
                   "latent_attn: bad arguments (value width <= 512)");
     MI355_REQUIRE(dt == MI355_DT_BF16 || dt == MI355_DT_F32, "latent_attn: bad dtype");
@@ -418,6 +489,10 @@ extern "C" int mi355_latent_attn(int n_seq, int max_new, int H, int hm, int D1, 
     MI355_REQUIRE(hm >= 1 && hm <= AM && AM % hm == 0 && (hm == 1 || (k1_hs == 0 && v_hs == 0) || kv_rep % hm == 0),
                   "latent_attn: several heads per tile (a power of two <= 32) need shared keys and values (head stride 0, or one key / value head for the tile's heads)");
     MI355_REQUIRE(!use_mfma || dt == MI355_DT_BF16, "latent_attn: the MFMA path takes bf16 keys and values");
+    MI355_REQUIRE(softcap >= 0.f && pool >= 0, "latent_attn: bad softcap or pool");
+    MI355_REQUIRE(pool == 0 || (window > 0 && keep_first == 0 && D2 == 0 && PK && PV && pool_row0 && ldp >= (int64_t)((H - 1) / kv_rep) * k1_hs + D1 &&
+                                ldp >= (int64_t)((H - 1) / kv_rep) * v_hs + DV),
+                  "latent_attn: pooled blocks need a window, one-part keys and the pooled rows (laid out like the key / value rows)");
     MI355_REQUIRE(q_row0 && n_new && past && k1_row0 && k2_row0 && v_row0, "latent_attn: sequence descriptors missing");
     MI355_REQUIRE(ldq >= (int64_t)(H - 1) * q_hs + D1 + D2 && ldo >= (int64_t)(H - 1) * o_hs + DV && ldk1 >= (int64_t)((H - 1) / kv_rep) * k1_hs + D1 && ldv >= (int64_t)((H - 1) / kv_rep) * v_hs + DV &&
                       (D2 == 0 || ldk2 >= D2),
@@ -430,6 +505,7 @@ extern "C" int mi355_latent_attn(int n_seq, int max_new, int H, int hm, int D1, 
     p.q_row0 = q_row0, p.n_new = n_new, p.past = past, p.k1_row0 = k1_row0, p.k2_row0 = k2_row0, p.v_row0 = v_row0;
     p.scale = scale;
     p.kv_rep = kv_rep, p.window = window, p.keep_first = keep_first;
+    p.softcap = softcap, p.sink = sink, p.pool = pool, p.PK = PK, p.PV = PV, p.ldp = ldp, p.pool_row0 = pool_row0;
     p.splits = 1, p.ws = nullptr;
     const bool mfma = use_mfma && D1 + D2 <= 320 && DV <= 256;  // what the MFMA kernel keeps in registers; larger heads take the FMA path
     const int tm = (mfma ? MQ : AM) / hm;
@@ -445,7 +521,8 @@ extern "C" int mi355_latent_attn(int n_seq, int max_new, int H, int hm, int D1, 
     }
     if (mfma) {
         const int vec_ok = D1 % 8 == 0 && D2 % 8 == 0 && DV % 8 == 0 && ldk1 % 8 == 0 && ldk2 % 8 == 0 && ldv % 8 == 0 && k1_hs % 8 == 0 && v_hs % 8 == 0 &&
-                           ((uintptr_t)K1 & 15) == 0 && ((uintptr_t)K2 & 15) == 0 && ((uintptr_t)V & 15) == 0;
+                           ((uintptr_t)K1 & 15) == 0 && ((uintptr_t)K2 & 15) == 0 && ((uintptr_t)V & 15) == 0 &&
+                           (pool == 0 || (ldp % 8 == 0 && ((uintptr_t)PK & 15) == 0 && ((uintptr_t)PV & 15) == 0));
         const int DK = D1 + D2;
         if (DK <= 64) launch_mfma<8>(p, grid, vec_ok, ST(stream));
         else if (DK <= 128) launch_mfma<16>(p, grid, vec_ok, ST(stream));

@@ -241,10 +241,11 @@ __device__ __forceinline__ void turn_pair(float u, float v, float ang, float& ou
 }
 
 // Latent key/value row of token t: src[t] = [rank values | rot values].  dst row dst_row[t] of the cache receives
-// [RMSNorm(first rank) * w | rotate(last rot)] (the first `dims` of the rot part turn, the rest pass).
+// [RMSNorm(first rank) * w | rotate(last rot)] (the first `dims` of the rot part turn, the rest pass).  layout 0: pair i = entries (2i, 2i+1);
+// layout 1: pair i = entries (i, i + dims/2).
 __global__ __launch_bounds__(256) void latent_kv_append_kernel(int64_t T, int rank, int rot, const void* __restrict__ src, int src_dt, int64_t lds_, const float* __restrict__ w,
                                                                float eps, const int* __restrict__ pos, const int* __restrict__ dst_row, const float* __restrict__ freq,
-                                                               int dims, void* __restrict__ cache, int cache_dt, int64_t ldc) {
+                                                               int dims, int layout, void* __restrict__ cache, int cache_dt, int64_t ldc) {
     const int lane = threadIdx.x & 63;
     for (int64_t t = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6); t < T; t += (int64_t)gridDim.x * 4) {
         const int64_t so = t * lds_, d0 = (int64_t)dst_row[t] * ldc;
@@ -256,6 +257,16 @@ __global__ __launch_bounds__(256) void latent_kv_append_kernel(int64_t T, int ra
         const float r = 1.0f / sqrtf(wave_sum(s) / (float)rank + eps);
         for (int i = lane; i < rank; i += 64) st_dt(cache, cache_dt, d0 + i, ld_dt(src, src_dt, so + i) * r * w[i]);
         const float p = (float)pos[t];
+        if (layout == 1) {
+            for (int i = dims + lane; i < rot; i += 64) st_dt(cache, cache_dt, d0 + rank + i, ld_dt(src, src_dt, so + rank + i));
+            for (int i = lane; i < dims / 2; i += 64) {
+                float ou, ov;
+                turn_pair(ld_dt(src, src_dt, so + rank + i), ld_dt(src, src_dt, so + rank + i + dims / 2), p * freq[i], ou, ov);
+                st_dt(cache, cache_dt, d0 + rank + i, ou);
+                st_dt(cache, cache_dt, d0 + rank + i + dims / 2, ov);
+            }
+            continue;
+        }
         for (int i = lane; i < (rot + 1) / 2; i += 64) {
             const float u = ld_dt(src, src_dt, so + rank + 2 * i);
             const bool has_v = 2 * i + 1 < rot;
@@ -269,10 +280,10 @@ __global__ __launch_bounds__(256) void latent_kv_append_kernel(int64_t T, int ra
 }
 
 extern "C" int mi355_latent_kv_append(int64_t tokens, int rank, int rot, const void* src, int src_dt, int64_t ld, const float* w, float eps, const int* pos,
-                                      const int* dst_row, const float* freq, int dims, void* cache, int cache_dt, int64_t ldc, void* stream) {
-    MI355_REQUIRE(tokens > 0 && rank > 0 && rot >= 0 && src && w && pos && dst_row && cache && dt_ok(src_dt) && dt_ok(cache_dt), "latent_kv_append: bad arguments");
+                                      const int* dst_row, const float* freq, int dims, int layout, void* cache, int cache_dt, int64_t ldc, void* stream) {
+    MI355_REQUIRE(tokens > 0 && rank > 0 && rot >= 0 && src && w && pos && dst_row && cache && dt_ok(src_dt) && dt_ok(cache_dt) && (layout == 0 || layout == 1), "latent_kv_append: bad arguments");
     MI355_REQUIRE(ld >= rank + rot && ldc >= rank + rot && dims >= 0 && dims <= rot && dims % 2 == 0 && (dims == 0 || freq), "latent_kv_append: bad row sizes");
-    latent_kv_append_kernel<<<rows_grid(tokens, 4), 256, 0, ST(stream)>>>(tokens, rank, rot, src, src_dt, ld, w, eps, pos, dst_row, freq, dims, cache, cache_dt, ldc);
+    latent_kv_append_kernel<<<rows_grid(tokens, 4), 256, 0, ST(stream)>>>(tokens, rank, rot, src, src_dt, ld, w, eps, pos, dst_row, freq, dims, layout, cache, cache_dt, ldc);
     MI355_LAUNCH_CHECK("latent_kv_append");
     return 0;
 }

@@ -335,7 +335,13 @@ extern "C" int mi355_ragged_conv(int64_t tokens, int n_seq, int C, int taps, con
 // src[t] = [H query heads x d | G key heads x d | G value heads x dv] (+ bias).  Query and key heads: RMS norm over d with a weight shared by the heads
 // (absent: none), rotary on the first `dims` entries (layout 0: pairs (2i, 2i+1); 1: pairs (i, i + dims/2)), angle = pos * freq[i]; a query head is then
 // multiplied by qscale[h] and written as fp32 to q_out[t, h * d + .]; key and value heads go to cache row dst_row[t]: [G x d | G x dv] in dtype c_dt.
+// Query temperature (qt_every > 0): the query at position p is also multiplied by 1 + qt_coef * ln(floor((p + 1) / qt_every) + 1).  Value mixing
+// (vmix given): v <- (1 - lam) v + lam * vmix[t] before it is cached, vmix fp32 rows [G x dv] (another layer's values of the same tokens).
 struct QkvRowsArgs {
+    const float* vmix;
+    int64_t ldvm;
+    float lam, qt_coef;
+    int qt_every;
     const void* src;
     const float* bias;
     const float *qw, *kw, *qscale, *freq;
@@ -361,7 +367,12 @@ __global__ __launch_bounds__(256) void qkv_rows_kernel(int64_t T, QkvRowsArgs p)
         auto val = [&](int i) { return ldr_dt(p.src, p.src_dt, so + i) + (p.bias ? p.bias[col0 + i] : 0.f); };
         if (!is_q && !is_k) {
             const int64_t d0 = (int64_t)p.dst_row[t] * p.ldc + p.G * p.d + (hh - p.H - p.G) * p.dv;
-            for (int i = lane; i < n; i += 64) str_dt(p.cache, p.c_dt, d0 + i, val(i));
+            if (p.vmix) {
+                const int64_t m0 = t * p.ldvm + (hh - p.H - p.G) * p.dv;
+                for (int i = lane; i < n; i += 64) str_dt(p.cache, p.c_dt, d0 + i, (1.0f - p.lam) * val(i) + p.lam * p.vmix[m0 + i]);
+            } else {
+                for (int i = lane; i < n; i += 64) str_dt(p.cache, p.c_dt, d0 + i, val(i));
+            }
             continue;
         }
         const float* w = is_q ? p.qw : p.kw;
@@ -374,7 +385,8 @@ __global__ __launch_bounds__(256) void qkv_rows_kernel(int64_t T, QkvRowsArgs p)
             }
             r = 1.0f / sqrtf(wave_sum(s) / (float)n + p.eps);
         }
-        const float sc = is_q ? (p.qscale ? p.qscale[hh] : 1.0f) : 1.0f;
+        float sc = is_q ? (p.qscale ? p.qscale[hh] : 1.0f) : 1.0f;
+        if (is_q && p.qt_every > 0) sc *= 1.0f + p.qt_coef * logf((float)((p.pos[t] + 1) / p.qt_every + 1));
         const float ps = (float)p.pos[t];
         const int64_t qo = t * p.ldq + (int64_t)hh * p.d, ko = (int64_t)p.dst_row[t] * p.ldc + (int64_t)(hh - p.H) * p.d;
         auto put = [&](int i, float v) {
@@ -396,13 +408,16 @@ __global__ __launch_bounds__(256) void qkv_rows_kernel(int64_t T, QkvRowsArgs p)
 
 extern "C" int mi355_qkv_rows_append(int64_t tokens, int H, int G, int d, int dv, const void* src, int src_dt, int64_t ld_src, const float* bias, const float* qw,
                                      const float* kw, float eps, const float* qscale, int dims, int layout, const float* freq, const int* pos, const int* dst_row,
-                                     float* q_out, int64_t ldq, void* cache, int c_dt, int64_t ldc, void* stream) {
+                                     float* q_out, int64_t ldq, void* cache, int c_dt, int64_t ldc, float qt_coef, int qt_every, const float* vmix, int64_t ldvm,
+                                     float lam, void* stream) {
+    MI355_REQUIRE(qt_every >= 0 && (!vmix || ldvm >= (int64_t)G * dv), "qkv_rows_append: bad query temperature or value-mix rows");
     MI355_REQUIRE(tokens > 0 && H > 0 && G > 0 && d > 0 && dv > 0 && src && pos && dst_row && q_out && cache && rec_dt_ok(src_dt) && rec_dt_ok(c_dt), "qkv_rows_append: bad arguments");
     MI355_REQUIRE(dims >= 0 && dims % 2 == 0 && dims <= d && (dims == 0 || freq) && (layout == 0 || layout == 1), "qkv_rows_append: the rotated range must lie inside a head");
     MI355_REQUIRE(ld_src >= (int64_t)(H + G) * d + (int64_t)G * dv && ldq >= (int64_t)H * d && ldc >= (int64_t)G * (d + dv), "qkv_rows_append: rows too short");
     QkvRowsArgs p;
     p.src = src, p.bias = bias, p.qw = qw, p.kw = kw, p.qscale = qscale, p.freq = freq, p.pos = pos, p.dst_row = dst_row, p.q_out = q_out, p.cache = cache;
     p.lds_ = ld_src, p.ldq = ldq, p.ldc = ldc, p.src_dt = src_dt, p.c_dt = c_dt, p.H = H, p.G = G, p.d = d, p.dv = dv, p.dims = dims, p.layout = layout, p.eps = eps;
+    p.vmix = vmix, p.ldvm = ldvm, p.lam = lam, p.qt_coef = qt_coef, p.qt_every = qt_every;
     qkv_rows_kernel<<<rec_rows_grid(tokens * (H + 2 * G), 4), 256, 0, ST(stream)>>>(tokens, p);
     MI355_LAUNCH_CHECK("qkv_rows_append");
     return 0;

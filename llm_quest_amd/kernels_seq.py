@@ -1,7 +1,8 @@
-"""Python launchers of the ragged-batch serving kernels (csrc/seqmix.hip, csrc/bgemm.hip, csrc/latent_attn.hip, csrc/seqrec.hip): hashed-bigram embedding,
+"""Python launchers of the ragged-batch serving kernels (csrc/seqmix.hip, csrc/bgemm.hip, csrc/latent_attn.hip, csrc/seqrec.hip, csrc/seqsand.hip): hashed-bigram embedding,
 post-sum LayerNorm on an fp32 residual stream, latent key/value rows, rotary embedding in both pair layouts, two-part-key / grouped-query / windowed attention,
 gated linear attention and retention with carried state, the sigmoid and softmax routers and the grouped expert products (with gated epilogues), the residual
-sum with RMS norms in groups, short convolutions with carried inputs, query / key / value rows into a slot cache, the gated delta rule, gated activations.
+sum with RMS norms in groups, short convolutions with carried inputs, query / key / value rows into a slot cache, the gated delta rule, gated activations,
+the residual sum between two norms (sandwich norms), pooled key / value rows, xIELU and sigmoid output gates on rows.
 
 Activations are bf16 (serving mode: bf16 operands, fp32 accumulation) or fp32 (true 32-bit mode: every product is an fp32 FMA chain; the bf16
 weights are exactly representable and widened on load).  Whatever the mode, the residual stream, norm statistics, rotary angles, decays,
@@ -81,8 +82,9 @@ def rope_frequencies(dims, base, device):
     return torch.pow(torch.tensor(float(base), dtype=torch.float64), -2.0 * i / dims).to(F32).to(device)
 
 
-def latent_kv_append(src, rank, rot, w, eps, pos, dst_row, freq, dims, cache2d):
-    """src [tokens, rank + rot] -> rows ``dst_row`` of ``cache2d`` [rows, rank + rot]: RMSNorm on the latent, interleaved rotary on the shared key part."""
+def latent_kv_append(src, rank, rot, w, eps, pos, dst_row, freq, dims, cache2d, layout=0):
+    """src [tokens, rank + rot] -> rows ``dst_row`` of ``cache2d`` [rows, rank + rot]: RMSNorm on the latent, rotary on the shared key part (``layout`` 0:
+    neighbouring entries form a pair; 1: entry i pairs with entry i + dims / 2)."""
     L.require_gpu(src, w, pos, dst_row, freq, cache2d)
     _rows(src, "latent_kv_append(src)")
     _rows(cache2d, "latent_kv_append(cache)")
@@ -92,7 +94,7 @@ def latent_kv_append(src, rank, rot, w, eps, pos, dst_row, freq, dims, cache2d):
     if src.shape[1] != rank + rot or cache2d.shape[1] != rank + rot or w.dtype != F32 or w.numel() != rank or (dims and (freq.dtype != F32 or freq.numel() < dims // 2)):
         raise ValueError("latent_kv_append: operand sizes do not match rank / rot")
     L.call("mi355_latent_kv_append", T, rank, rot, L.ptr(src), _dt(src), src.stride(0), L.ptr(w), float(eps), L.ptr(pos), L.ptr(dst_row), L.ptr(freq), int(dims),
-           L.ptr(cache2d), _dt(cache2d), cache2d.stride(0))
+           int(layout), L.ptr(cache2d), _dt(cache2d), cache2d.stride(0))
 
 
 def rope_heads(src, H, n, src_hs, src_off, dst, dst_hs, dst_off, rot_start, dims, freq, pos, layout=0):
@@ -243,12 +245,26 @@ def attn_key_splits(n_seq, head_tiles, max_new, hm, max_keys):
     return max(1, min(-(-max_keys // 256), 32, 256 // tiles))
 
 
-def latent_attn(q, k1, k2, v, out, H, hm, D1, D2, DV, q_hs, k1_hs, v_hs, o_hs, desc, max_new, scale, max_keys=0, kv_rep=1, window=0, keep_first=0):
+def latent_attn(q, k1, k2, v, out, H, hm, D1, D2, DV, q_hs, k1_hs, v_hs, o_hs, desc, max_new, scale, max_keys=0, kv_rep=1, window=0, keep_first=0, softcap=0.0,
+                sink=None, pool=0, pooled=None, pool_row0=None):
     """Two-part-key causal attention over a ragged batch.  ``desc`` = (q_row0, n_new, past, k1_row0, k2_row0, v_row0) int32 [n_seq] each.  ``max_keys``
     (the longest sequence's keys, if the caller knows it) lets one-token steps over long caches spread a tile's keys over several workgroups.
     ``kv_rep``: query heads per key / value head (strides per key / value head).  ``window`` > 0: a query sees a key only ``window`` positions back, or
-    among the first ``keep_first`` of the sequence."""
-    L.require_gpu(q, k1, k2, v, out, *desc)
+    among the first ``keep_first`` of the sequence.  ``softcap`` > 0: scores pass cap * tanh(score / cap).  ``sink`` (fp32 [H]): exp(sink[h]) joins head h's
+    denominator.  ``pool`` > 0: ``pooled`` = (pooled keys, pooled values), views laid out like ``k1`` / ``v`` with one mean row per ``pool`` tokens, first row
+    of every sequence in ``pool_row0`` (int32 [n_seq]); a query sees the blocks that lie wholly before its window."""
+    L.require_gpu(q, k1, k2, v, out, sink, pool_row0, *desc)
+    pk = pv = None
+    if pool:
+        pk, pv = pooled
+        L.require_gpu(q, pk, pv)
+        _rows(pk, "latent_attn(pooled keys)")
+        _rows(pv, "latent_attn(pooled values)")
+        _i32(pool_row0, "latent_attn(pool_row0)", desc[0].numel())
+        if pk.dtype != v.dtype or pv.dtype != v.dtype or pk.stride(0) != pv.stride(0):
+            raise ValueError("latent_attn: pooled rows share the dtype of keys / values and one row pitch")
+    if sink is not None and (sink.dtype != F32 or not sink.is_contiguous() or sink.numel() != H):
+        raise ValueError("latent_attn: sink fp32 [H]")
     for t, n in ((q, "q"), (k1, "k1"), (v, "v"), (out, "out")):
         _rows(t, f"latent_attn({n})")
     if q.dtype != F32 or k1.dtype != v.dtype or out.dtype != v.dtype or (k2 is not None and k2.dtype != v.dtype):
@@ -267,7 +283,8 @@ def latent_attn(q, k1, k2, v, out, H, hm, D1, D2, DV, q_hs, k1_hs, v_hs, o_hs, d
             ws = torch.empty(n_seq * head_tiles * -(-max_new * hm // 128) * splits * 128 * (2 + dvp), dtype=F32, device=v.device)
     L.call("mi355_latent_attn", n_seq, max_new, H, hm, D1, D2, DV, L.ptr(q), q.stride(0), q_hs, L.ptr(k1), k1.stride(0), k1_hs, L.ptr(k2), 0 if k2 is None else k2.stride(0),
            L.ptr(v), v.stride(0), v_hs, L.ptr(out), out.stride(0), o_hs, _dt(v), *[L.ptr(t) for t in desc], float(scale), 1 if mfma else 0, splits, L.ptr(ws),
-           0 if ws is None else ws.numel(), int(kv_rep), int(window), int(keep_first))
+           0 if ws is None else ws.numel(), int(kv_rep), int(window), int(keep_first), float(softcap or 0.0), L.ptr(sink), int(pool), L.ptr(pk), L.ptr(pv),
+           0 if pk is None else pk.stride(0), L.ptr(pool_row0))
     return out
 
 
@@ -326,9 +343,18 @@ def ragged_conv(x, w, state, row_seq, seq_off, slot, act=False, residual=False, 
     return y
 
 
-def qkv_rows_append(src, H, G, d, dv, bias, qw, kw, eps, qscale, dims, layout, freq, pos, dst_row, cache2d):
-    """Rows [H x d | G x d | G x dv] -> fp32 queries [tokens, H * d] (bias, head norm, rotation, per-head scale) and key / value rows of ``cache2d``."""
-    L.require_gpu(src, bias, qw, kw, qscale, freq, pos, dst_row, cache2d)
+def qkv_rows_append(src, H, G, d, dv, bias, qw, kw, eps, qscale, dims, layout, freq, pos, dst_row, cache2d, q_temp=None, vmix=None, lam=0.0):
+    """Rows [H x d | G x d | G x dv] -> fp32 queries [tokens, H * d] (bias, head norm, rotation, per-head scale) and key / value rows of ``cache2d``.
+    ``q_temp`` = (coef, every): the query at position p is also multiplied by 1 + coef * ln(floor((p + 1) / every) + 1).  ``vmix`` (fp32 [tokens, G * dv],
+    any row pitch): the cached value is (1 - lam) v + lam * vmix."""
+    L.require_gpu(src, bias, qw, kw, qscale, freq, pos, dst_row, cache2d, vmix)
+    if vmix is not None:
+        _rows(vmix, "qkv_rows_append(vmix)")
+        if vmix.dtype != F32 or tuple(vmix.shape) != (src.shape[0], G * dv):
+            raise ValueError(f"qkv_rows_append: the rows to mix in are fp32 [{src.shape[0]}, {G * dv}]")
+    coef, every = (float(q_temp[0]), int(q_temp[1])) if q_temp else (0.0, 0)
+    if q_temp and every < 1:
+        raise ValueError("qkv_rows_append: the query temperature's step is a positive number of positions")
     _rows(src, "qkv_rows_append(src)")
     _rows(cache2d, "qkv_rows_append(cache)")
     T = src.shape[0]
@@ -341,7 +367,8 @@ def qkv_rows_append(src, H, G, d, dv, bias, qw, kw, eps, qscale, dims, layout, f
     _i32(dst_row, "qkv_rows_append(dst_row)", T)
     q = torch.empty((T, H * d), dtype=F32, device=src.device)
     L.call("mi355_qkv_rows_append", T, H, G, d, dv, L.ptr(src), _dt(src), src.stride(0), L.ptr(bias), L.ptr(qw), L.ptr(kw), float(eps), L.ptr(qscale), int(dims), int(layout),
-           L.ptr(freq), L.ptr(pos), L.ptr(dst_row), L.ptr(q), q.stride(0), L.ptr(cache2d), _dt(cache2d), cache2d.stride(0))
+           L.ptr(freq), L.ptr(pos), L.ptr(dst_row), L.ptr(q), q.stride(0), L.ptr(cache2d), _dt(cache2d), cache2d.stride(0), coef, every, L.ptr(vmix),
+           0 if vmix is None else vmix.stride(0), float(lam))
     return q
 
 
@@ -395,4 +422,64 @@ def glu_rows(x, kind, limit=0.0, out_dtype=None):
     F = x.shape[1] // 2
     out = torch.empty((x.shape[0], F), dtype=out_dtype or x.dtype, device=x.device)
     L.call("mi355_glu_rows", x.shape[0], F, L.ptr(x), _dt(x), x.stride(0), int(kind), float(limit), L.ptr(out), _dt(out), out.stride(0))
+    return out
+
+
+def sandwich_rmsnorm(x, eps, y=None, w_post=None, w_next=None, out_dtype=None, x_out=None):
+    """The residual sum between two norms: v = x + RMSNorm(y) * w_post (``y`` None: v = x); ``x_out`` (True: a new tensor; or x itself; or None) receives v;
+    with ``w_next`` the normed row RMSNorm(v) * w_next is returned in ``out_dtype``.  x fp32, weights fp32 [width].  Returns (x_out or None, normed or None)."""
+    L.require_gpu(x, y, w_post, w_next)
+    _rows(x, "sandwich_rmsnorm(x)")
+    T, width = x.shape
+    if x.dtype != F32 or not x.is_contiguous():
+        raise ValueError("sandwich_rmsnorm: x contiguous fp32 [tokens, width]")
+    if y is not None:
+        _rows(y, "sandwich_rmsnorm(y)")
+        if tuple(y.shape) != (T, width) or w_post is None:
+            raise ValueError(f"sandwich_rmsnorm: the sublayer output is [{T}, {width}] and comes with its norm weight")
+    for w in (w_post, w_next):
+        if w is not None and (w.dtype != F32 or w.numel() != width or not w.is_contiguous()):
+            raise ValueError("sandwich_rmsnorm: weight fp32 [width]")
+    if x_out is True:
+        x_out = torch.empty_like(x)
+    out = torch.empty((T, width), dtype=out_dtype or F32, device=x.device) if w_next is not None else None
+    L.call("mi355_sandwich_rmsnorm", T, width, L.ptr(x), L.ptr(y), 0 if y is None else _dt(y), 0 if y is None else y.stride(0), L.ptr(w_post), L.ptr(x_out), L.ptr(w_next),
+           float(eps), L.ptr(out), 0 if out is None else _dt(out))
+    return x_out, out
+
+
+def pool_rows_update(cache2d, pooled2d, pool, cache_row0, pool_row0, past, n_new, max_blocks):
+    """Every block of ``pool`` cache rows that this step completed gets its mean row in ``pooled2d`` (block b of sequence s = row pool_row0[s] + b).
+    ``max_blocks``: the most blocks one sequence completes in this step (the host knows the lengths); 0 launches nothing."""
+    if max_blocks <= 0:
+        return
+    L.require_gpu(cache2d, pooled2d, cache_row0, pool_row0, past, n_new)
+    _rows(cache2d, "pool_rows_update(cache)")
+    _rows(pooled2d, "pool_rows_update(pooled)")
+    n_seq = past.numel()
+    for t in (cache_row0, pool_row0, past, n_new):
+        _i32(t, "pool_rows_update(desc)", n_seq)
+    if cache2d.shape[1] != pooled2d.shape[1]:
+        raise ValueError("pool_rows_update: pooled rows are as wide as the cache rows")
+    L.call("mi355_pool_rows_update", n_seq, int(max_blocks), cache2d.shape[1], int(pool), L.ptr(cache2d), _dt(cache2d), cache2d.stride(0), L.ptr(pooled2d), _dt(pooled2d),
+           pooled2d.stride(0), L.ptr(cache_row0), L.ptr(pool_row0), L.ptr(past), L.ptr(n_new))
+
+
+ACT_XIELU, ACT_SIGMOID_GATE = 0, 1
+
+
+def act_rows(x, kind, params=None, gate=None, out_dtype=None):
+    """``ACT_XIELU``: z > 0: softplus(p) z^2 + z / 2, z <= 0: (1/2 + softplus(q)) (exp(z) - 1 - z) + z / 2 with ``params`` = fp32 [p, q];
+    ``ACT_SIGMOID_GATE``: x * sigmoid(gate).  Rows may be views with any pitch."""
+    L.require_gpu(x, params, gate)
+    _rows(x, "act_rows(x)")
+    if kind == ACT_XIELU and (params is None or params.dtype != F32 or params.numel() != 2 or not params.is_contiguous()):
+        raise ValueError("act_rows: xIELU takes fp32 [p, q]")
+    if kind == ACT_SIGMOID_GATE:
+        _rows(gate, "act_rows(gate)")
+        if gate.shape != x.shape:
+            raise ValueError("act_rows: the gate has x's shape")
+    out = torch.empty(x.shape, dtype=out_dtype or x.dtype, device=x.device)
+    L.call("mi355_act_rows", x.shape[0], x.shape[1], L.ptr(x), _dt(x), x.stride(0), L.ptr(gate), 0 if gate is None else _dt(gate), 0 if gate is None else gate.stride(0),
+           int(kind), L.ptr(params), L.ptr(out), _dt(out), out.stride(0))
     return out

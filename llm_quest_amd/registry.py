@@ -34,8 +34,15 @@ def _mepatar(model_dir, act_dtype, device):
     return load_mepatar(model_dir, act_dtype, device)
 
 
+def _mopalorn(model_dir, act_dtype, device):
+    from llm_quest_amd.mopalorn.mopalorn_weight_loading import load_mopalorn
+
+    return load_mopalorn(model_dir, act_dtype, device)
+
+
 register("Gemepel", _gemepel)
 register("Mepatar", _mepatar)
+register("Mopalorn", _mopalorn)
 
 
 def load_model(model_dir, dtype="bfloat16", device="cuda"):

@@ -148,7 +148,9 @@ class SlotStateCache:
       * ``("shared", j)``    -- the layer reads layer j's rows and stores nothing;
       * ``("state", shape)`` -- a fixed-size fp32 state ``[slots, *shape]`` (the matrix state of linear attention), zeroed when a slot is opened;
       * ``{"rows": width or None, "states": {name: shape}}`` -- both at once, with several named fp32 states (``state(i, name)``): a layer that caches
-        key / value rows and carries the last inputs of short convolutions, or a recurrent state next to its convolutions' inputs;
+        key / value rows and carries the last inputs of short convolutions, or a recurrent state next to its convolutions' inputs; with ``"pool": P``
+        the layer also keeps one row per block of P tokens (``pooled2d(i)``, ``[slots, ceil(capacity / P), width]``: the mean rows of attention that sees old
+        tokens block-wise), which grow with the rows;
       * ``None``             -- nothing.
     Besides, per slot: the length so far and the last token (the embedding of some designs looks one token back).  Growth follows ``KVCache``: the row
     capacity starts at what the first sequences need plus ``initial_chunk_size`` and grows by whole ``chunk_size`` steps up to ``context_len``; slots double."""
@@ -161,6 +163,7 @@ class SlotStateCache:
         self.slots = max(1, int(slots))
         self.capacity = min(self.context_len, int(capacity))
         self.rows = [None] * len(self.layer_specs)
+        self.pooled = [None] * len(self.layer_specs)  # layers with a "pool" entry: [slots, ceil(capacity / pool), width]
         self.states = [None] * len(self.layer_specs)
         self.named = [{} for _ in self.layer_specs]  # layer -> name -> fp32 [slots, *shape]
         self.length = [0] * self.slots
@@ -196,7 +199,19 @@ class SlotStateCache:
                 n = min(old.shape[0], self.slots)
                 new[:n, : old.shape[1]].copy_(old[:n])
             self.rows[i] = new
+            pool = self.pool_size(i)
+            if pool:
+                old = self.pooled[i]
+                new = torch.zeros((self.slots, -(-capacity // pool), width), dtype=self.dtype, device=self.device)
+                if old is not None:
+                    n = min(old.shape[0], self.slots)
+                    new[:n, : old.shape[1]].copy_(old[:n])
+                self.pooled[i] = new
         self.capacity = capacity
+
+    def pool_size(self, layer_idx):
+        spec = self.layer_specs[layer_idx]
+        return int(spec.get("pool") or 0) if isinstance(spec, dict) else 0
 
     def _grow_slots(self):
         add = self.slots
@@ -274,6 +289,14 @@ class SlotStateCache:
     def rows2d(self, layer_idx):
         r = self.rows[self.source(layer_idx)]
         return r.view(r.shape[0] * r.shape[1], r.shape[2])
+
+    def pooled2d(self, layer_idx):
+        """The layer's pooled rows as [slots * blocks per slot, width]; block b of a slot is row slot * pool_capacity(layer) + b."""
+        r = self.pooled[layer_idx]
+        return r.view(r.shape[0] * r.shape[1], r.shape[2])
+
+    def pool_capacity(self, layer_idx):
+        return self.pooled[layer_idx].shape[1]
 
     def state(self, layer_idx, name=None):
         return self.states[layer_idx] if name is None else self.named[layer_idx][name]
