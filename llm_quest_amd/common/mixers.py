@@ -177,8 +177,9 @@ class LatentAttention(_Frozen):
             while hm < min(H, 32):
                 hm *= 2
             ol = torch.empty((T, H * R), dtype=st.act_dtype, device=h.device)
-            S.latent_attn(qf, cache2d, cache2d[:, R:], cache2d, ol, H, hm, R, dr, R, R + dr, 0, 0, R,
-                          (st.q_row0, st.n_new, st.past, st.cache_row0, st.cache_row0, st.cache_row0), st.max_new, self.scale, max_keys=st.max_keys, window=win)
+            for v0 in range(0, R, 512):  # the attention takes values up to 512 wide: a wider latent goes in parts (the scores are the same every time)
+                S.latent_attn(qf, cache2d, cache2d[:, R:], cache2d[:, v0:], ol[:, v0:], H, hm, R, dr, min(512, R - v0), R + dr, 0, 0, R,
+                              (st.q_row0, st.n_new, st.past, st.cache_row0, st.cache_row0, st.cache_row0), st.max_new, self.scale, max_keys=st.max_keys, window=win)
             ctx = torch.empty((T, H * dv), dtype=st.act_dtype, device=h.device)
             S.bgemm(ol, self.w_ukv[H * dn :], ctx, T, dv, R, batch=H, lda=H * R, a_bs=R, sbn=R, sbk=1, b_bs=dv * R, ldc=H * dv, c_bs=dv)
         if self.gate:

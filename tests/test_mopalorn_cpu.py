@@ -1,0 +1,125 @@
+"""CPU checks of the Mopalorn serving path that need no GPU: the plain oracle's mechanisms against closed forms and against each other, the configuration
+reader, the checkpoint loader's fused layouts, the pooled rows of the slot cache and the step descriptors."""
+
+import math
+
+import pytest
+import torch
+
+from oracle import mopalorn as O
+from tests import mopalorn_util as U
+
+F64 = torch.float64
+
+
+def test_rms_norm_has_eps_inside_the_root():
+    x, w = torch.tensor([[3.0, 4.0]], dtype=F64), torch.tensor([2.0, 0.5], dtype=F64)
+    assert torch.allclose(O.rms_norm(x, w, 0.5), x / math.sqrt(12.5 + 0.5) * w)
+
+
+def test_rotate_half_pairs_entry_i_with_i_plus_half_and_keeps_the_rest():
+    x = torch.arange(2 * 1 * 8, dtype=F64).reshape(2, 1, 8) + 1
+    y = O.rotary_half(x, 4, 100.0)
+    assert torch.equal(y[0], x[0]) and torch.equal(y[:, :, 4:], x[:, :, 4:])
+    for i, (a, b) in enumerate([(0, 2), (1, 3)]):
+        ang = 100.0 ** (-2.0 * i / 4)
+        assert math.isclose(float(y[1, 0, a]), float(x[1, 0, a]) * math.cos(ang) - float(x[1, 0, b]) * math.sin(ang))
+        assert math.isclose(float(y[1, 0, b]), float(x[1, 0, b]) * math.cos(ang) + float(x[1, 0, a]) * math.sin(ang))
+    assert torch.allclose(O.rotary_half(x, 4, 100.0, first_position=5)[0], O.rotary_half(torch.cat([x[:1]] * 6), 4, 100.0)[5])
+
+
+def test_query_temperature_steps_where_p_plus_one_is_a_multiple():
+    t = O.query_temperature(20, 0.4, 8, F64)
+    assert torch.all(t[:7] == 1.0) and math.isclose(float(t[7]), 1 + 0.4 * math.log(2)) and t[14] == t[7] and math.isclose(float(t[15]), 1 + 0.4 * math.log(3))
+
+
+def test_window_and_pooled_block_edges():
+    assert O.window_keys(10, 4) == [7, 8, 9, 10] and O.window_keys(2, 4) == [0, 1, 2] and O.window_keys(3, 0) == [0, 1, 2, 3]
+    k = torch.arange(40, dtype=F64).reshape(40, 1, 1)
+    # window 4, pool 3: block b is seen once its last token 3 b + 2 <= i - 4
+    for i, n in ((5, 0), (6, 1), (8, 1), (9, 2), (12, 3)):
+        pk, pv = O.pooled_blocks(k, k, i, 4, 3)
+        assert pk.shape[0] == n
+        assert torch.equal(pk.flatten(), torch.tensor([3.0 * b + 1 for b in range(n)], dtype=F64))
+    # tokens that left the window whose block is not complete are seen by nobody: query 8 sees tokens 5..8 and block 0 (tokens 0..2), not 3, 4
+    T = 9
+    q = torch.zeros(T, 1, 2, dtype=F64)
+    kk = torch.zeros(T, 1, 2, dtype=F64)
+    v = torch.eye(T, dtype=F64).reshape(T, 1, T)
+    out = O.softmax_attention(q, kk, v, 1.0, lambda i: O.window_keys(i, 4), extra=lambda i: O.pooled_blocks(kk, v, i, 4, 3))[8, 0]
+    assert torch.allclose(out, torch.tensor([1 / 15] * 3 + [0, 0] + [1 / 5] * 4, dtype=F64))
+
+
+def test_sink_joins_the_denominator_only_and_cap_saturates():
+    q, k, v = torch.ones(1, 1, 1, dtype=F64), torch.ones(1, 1, 1, dtype=F64), torch.full((1, 1, 1), 7.0, dtype=F64)
+    out = O.softmax_attention(q, k, v, 2.0, lambda i: [0], sink=torch.tensor([0.5], dtype=F64))
+    assert math.isclose(float(out), 7.0 * math.exp(2.0) / (math.exp(2.0) + math.exp(0.5)))
+    assert math.isclose(float(O.soft_cap(torch.tensor(1e3, dtype=F64), 5.0)), 5.0) and math.isclose(float(O.soft_cap(torch.tensor(0.01, dtype=F64), 5.0)), 0.01, rel_tol=1e-5)
+
+
+def test_xielu_is_continuous_with_slope_one_half_at_zero():
+    p, q = torch.tensor(0.3, dtype=F64), torch.tensor(-0.2, dtype=F64)
+    z = torch.tensor([-1e-6, 0.0, 1e-6], dtype=F64)
+    y = O.xielu(z, p, q)
+    assert float(y[1]) == 0.0 and math.isclose(float(y[2] - y[0]) / 2e-6, 0.5, rel_tol=1e-5)
+    sp = math.log1p(math.exp(0.3))
+    assert math.isclose(float(O.xielu(torch.tensor(2.0, dtype=F64), p, q)), sp * 4 + 1.0)
+    sq = math.log1p(math.exp(-0.2))
+    assert math.isclose(float(O.xielu(torch.tensor(-2.0, dtype=F64), p, q)), (0.5 + sq) * (math.exp(-2.0) - 1 + 2.0) - 1.0)
+
+
+def test_value_mixing_takes_the_first_mixing_layers_values():
+    cs = U.make_config([(U.capped(v_mix=False), None), (U.pooled(), None), (U.capped(), None)])
+    w = U.make_weights(cs, 0)
+    assert "l0.mix.vmix" not in w and "l1.mix.vmix" in w
+    toks = list(range(30))
+    base = O.forward(toks, w, cs[0])
+    w2 = dict(w)
+    w2["l1.mix.vmix"] = torch.tensor(0.9, dtype=torch.bfloat16)  # the first mixing layer's own number is unused
+    assert torch.equal(O.forward(toks, w2, cs[0]), base)
+    w2["l2.mix.vmix"] = torch.tensor(0.9, dtype=torch.bfloat16)
+    assert not torch.allclose(O.forward(toks, w2, cs[0]), base)
+
+
+def test_config_reader_and_loader_layouts():
+    from llm_quest_amd.mopalorn.mopalorn_model import MopalornConfig, MopalornModel
+    from llm_quest_amd.mopalorn.mopalorn_weight_loading import load_mopalorn_state
+
+    cs = U.make_config(U.default_layers())
+    w = U.make_weights(cs, 3)
+    c = MopalornConfig(cs[0])
+    assert c.v_mix == [None, "first", None, "mix", None, "mix"] and c.logit_scale == 0.8
+    m = load_mopalorn_state(MopalornModel(c, sinks={i for i, s in enumerate(cs[1]) if s}), w)
+    la, pa, ca = m.blocks[0].mixer, m.blocks[1].mixer, m.blocks[3].mixer
+    nq = w["l0.mix.q"].shape[0]
+    assert torch.equal(la.w_down[:nq], w["l0.mix.q"]) and torch.equal(la.w_down[nq : nq + 64], w["l0.mix.dkv"]) and torch.equal(la.w_down[nq + 64 :], w["l0.mix.g"])
+    assert torch.equal(la.w_ukv, torch.cat([w["l0.mix.uk"], w["l0.mix.uv"]])) and la.window == 11 and la.rot_layout == 1 and la.gate
+    assert pa.pool == 5 and pa.window == 13 and pa.sink is not None and pa.lam is None and pa.v_mix == "first" and m.blocks[5].mixer.sink is None
+    assert ca.q_temp == (0.7, 9) and ca.softcap == 6.0 and ca.window == 0 and float(ca.lam) == float(w["l3.mix.vmix"])
+    assert m.blocks[2].ff is None and torch.equal(m.blocks[0].ff.act, w["l0.mlp.act"])
+    assert m.blocks[1].cache_spec() == {"rows": 2 * (24 + 40), "states": {}, "pool": 5}
+    bad = U.make_config([(U.pooled(), None), (U.capped(vdim=24), None)])
+    with pytest.raises(ValueError):
+        MopalornConfig(bad[0])
+    with pytest.raises(ValueError):
+        MopalornConfig({**cs[0], "architecture": "Other"})
+
+
+def test_registry_knows_the_design():
+    from llm_quest_amd import registry
+
+    assert "Mopalorn" in registry.architectures()
+
+
+def test_slot_cache_keeps_pooled_rows_through_growth():
+    from llm_quest_amd.utils import SlotStateCache
+
+    c = SlotStateCache([{"rows": 6, "pool": 4, "states": {}}, ("rows", 3)], 1000, "cpu", torch.float32, slots=1, capacity=10)
+    assert c.pool_size(0) == 4 and c.pool_size(1) == 0 and c.pool_capacity(0) == 3 and c.pooled[1] is None
+    c.pooled[0][0, 2] = 7.0
+    c.rows[0][0, 9] = 5.0
+    a, b = c.open("a"), c.open("b")  # a second slot: both buffers are laid out anew
+    c.reserve(30)
+    assert c.capacity >= 30 and c.pool_capacity(0) == -(-c.capacity // 4) and c.slots == 2
+    assert float(c.pooled[0][a, 2, 0]) == 7.0 and float(c.rows[0][a, 9, 0]) == 5.0 and float(c.pooled[0][b].abs().max()) == 0.0
+    assert c.pooled2d(0).shape == (2 * c.pool_capacity(0), 6)

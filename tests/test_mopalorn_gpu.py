@@ -1,0 +1,492 @@
+"""GPU tests of the Mopalorn serving path against the plain oracle (oracle/mopalorn.py): each mechanism's kernel or module alone, then the model through the
+registry, the slot cache and the ragged-batch scheduler -- whole prompts, token-by-token decoding, portions, unequal batches, reused slots, keys at the
+windows' and the pooled blocks' edges, odd sizes, greedy generation, the trace replay program.  fp32 mode is held to fp32 rounding; bf16 mode to a few
+bf16 roundings of the logits' scale."""
+
+import pytest
+import torch
+
+from oracle import mopalorn as O
+from tests import mopalorn_util as U
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+F32, F64, BF16, I32 = torch.float32, torch.float64, torch.bfloat16, torch.int32
+TOL = {"float32": 3e-5, "bfloat16": 8e-2}
+
+
+def dev_i32(x):
+    return torch.tensor(x, dtype=I32).to(DEV)
+
+
+def row_err(got, want):
+    """The worst row's rms of the difference (mean removed) over the rms of the wanted rows."""
+    got, want = got.detach().double().cpu(), want.detach().double().cpu()
+    d = got - want
+    d = d - d.mean(-1, keepdim=True)
+    return (d.pow(2).mean(-1).sqrt() / want.pow(2).mean().sqrt()).max().item()
+
+
+def tokens(n, vocab, seed):
+    g = torch.Generator().manual_seed(seed)
+    return torch.randint(0, vocab, (n,), generator=g).tolist()
+
+
+@pytest.fixture(scope="module")
+def checkpoint(tmp_path_factory):
+    cs = U.make_config(U.default_layers())
+    w = U.make_weights(cs, 11)
+    return U.save(str(tmp_path_factory.mktemp("mopalorn")), cs, w), cs[0], w
+
+
+@pytest.fixture(scope="module")
+def models(checkpoint):
+    from llm_quest_amd import registry
+
+    folder, cfg, w = checkpoint
+    return {dt: registry.load_model(folder, dt, DEV) for dt in ("float32", "bfloat16")}, cfg, w
+
+
+_oracle_cache = {}
+
+
+def oracle(cfg, w, toks, layers=False):
+    key = (id(w), tuple(toks), layers)
+    if key not in _oracle_cache:
+        _oracle_cache[key] = O.forward(toks, w, cfg, F64, return_layers=layers)
+    return _oracle_cache[key]
+
+
+def batch_of(model, **kw):
+    from llm_quest_amd.generate import RaggedBatch
+
+    return RaggedBatch(model, **kw)
+
+
+# ------------------------------------------------------------------------------------------------------------------- the model through the scheduler
+@pytest.mark.parametrize("dt", ["float32", "bfloat16"])
+def test_whole_prompt_every_layer(models, dt):
+    ms, cfg, w = models
+    toks = tokens(70, cfg["vocab"], 1)
+    want, layers = oracle(cfg, w, toks, layers=True)
+    b = batch_of(ms[dt])
+    got, got_layers = b.step([("a", toks)], [list(range(len(toks)))], return_layers=True)
+    assert len(got_layers) == len(layers)
+    for i, l in enumerate(got_layers):
+        assert row_err(l, layers[i]) < TOL[dt], f"residual stream after layer {i}"
+    assert row_err(got, want) < TOL[dt]
+
+
+@pytest.mark.parametrize("dt", ["float32", "bfloat16"])
+def test_token_by_token_from_the_first_token(models, dt):
+    """Every token alone: the first tokens see fewer keys than a window holds and no pooled block; blocks complete one token at a time."""
+    ms, cfg, w = models
+    toks = tokens(60, cfg["vocab"], 2)
+    want = oracle(cfg, w, toks)
+    b = batch_of(ms[dt])
+    got = torch.cat([b.step([("a", [t])]) for t in toks])
+    assert row_err(got, want) < TOL[dt]
+
+
+@pytest.mark.parametrize("dt", ["float32", "bfloat16"])
+def test_portions_of_several_sizes(models, dt):
+    """Portions down to one and two tokens: a portion may complete no pooled block, one, or several, and starts in the middle of one."""
+    ms, cfg, w = models
+    toks = tokens(90, cfg["vocab"], 3)
+    want = oracle(cfg, w, toks)
+    b = batch_of(ms[dt])
+    got, at = [], 0
+    for n in [7, 2, 2, 1, 33, 1, 9, 2, 33]:
+        got.append(b.step([("a", toks[at : at + n])], [list(range(n))]))
+        at += n
+    assert at == len(toks)
+    assert row_err(torch.cat(got), want) < TOL[dt]
+
+
+@pytest.mark.parametrize("dt", ["float32", "bfloat16"])
+def test_unequal_batch_equals_each_request_alone(models, dt):
+    ms, cfg, w = models
+    lens, tail = [1, 41, 17, 66], 9
+    seqs = [tokens(n + tail, cfg["vocab"], 10 + i) for i, n in enumerate(lens)]
+    alone = []
+    for s in seqs:
+        b = batch_of(ms[dt])
+        alone.append(b.step([("x", s)], [list(range(len(s)))]))
+    b = batch_of(ms[dt], slots=2)  # fewer slots than sequences: the cache grows
+    got = [[] for _ in seqs]
+    out = b.step([(i, s[: lens[i]]) for i, s in enumerate(seqs)], [list(range(n)) for n in lens])
+    at = 0
+    for i, n in enumerate(lens):
+        got[i].append(out[at : at + n])
+        at += n
+    live = list(range(len(seqs)))
+    for k in range(tail):
+        if k == 4:  # two requests leave early; the others go on
+            for i in (0, 2):
+                b.finish(i)
+                live.remove(i)
+        out = b.step([(i, [seqs[i][lens[i] + k]]) for i in live])
+        for j, i in enumerate(live):
+            got[i].append(out[j : j + 1])
+    for i, s in enumerate(seqs):
+        g = torch.cat(got[i])
+        ref = alone[i][: g.shape[0]]  # (alone, the whole request is one prompt: in bf16 its last tokens take the prompt form of the kernels, here the one-token form)
+        assert row_err(g, ref) < (1e-5 if dt == "float32" else 6e-2), f"request {i} in the batch differs from the request alone"
+        assert row_err(g, oracle(cfg, w, s)[: g.shape[0]]) < TOL[dt]
+
+
+def test_freed_slots_are_reused_without_leftovers(models):
+    """A long sequence leaves key / value rows and pooled rows behind; the next, shorter one takes its slot and must see none of them.  The cache starts
+    small, so rows and pooled rows also grow while a sequence is alive."""
+    ms, cfg, w = models
+    b = batch_of(ms["float32"], slots=1)
+    b.cache.initial_chunk_size, b.cache.chunk_size = 4, 8
+    long_, short = tokens(60, cfg["vocab"], 20), tokens(33, cfg["vocab"], 21)
+    b.step([("long", long_[:50])])
+    for t in long_[50:]:
+        b.step([("long", [t])])
+    b.finish("long")
+    got = [b.step([("short", short[:12])], [list(range(12))])] + [b.step([("short", [t])]) for t in short[12:]]
+    assert b.cache.reuses >= 1 and b.cache.slots == 1
+    assert row_err(torch.cat(got), oracle(cfg, w, short)) < TOL["float32"]
+
+
+def test_long_decoding_passes_windows_blocks_and_temperature_steps(models):
+    """Decoded tokens walk past every window (7 ... 13 keys), complete dozens of pooled blocks and cross many steps of the query temperature."""
+    ms, cfg, w = models
+    toks = tokens(200, cfg["vocab"], 30)
+    b = batch_of(ms["float32"])
+    b.step([("a", toks[:5])])
+    got = torch.cat([b.step([("a", [t])]) for t in toks[5:]])
+    assert row_err(got, oracle(cfg, w, toks)[5:]) < TOL["float32"]
+
+
+@pytest.mark.parametrize("dt", ["float32", "bfloat16"])
+def test_other_sizes_odd_and_one(tmp_path, dt):
+    """Sizes that are no multiples of 8 or of each other's, one head, a window of one key, a pool of one token (every token that left the window is its own
+    block), a pool larger than its window, a window that never closes, no pool, no sink, no cap, no query temperature, three query heads per key head, value
+    mixing that starts in a capped layer, a latent wider than the heads, a temperature step of one position, no scale on the logits."""
+    from llm_quest_amd import registry
+
+    plain = U.capped(heads=6, kv_heads=2, dim=12, vdim=20, v_mix=True)
+    del plain["mixer"]["q_temp"], plain["mixer"]["softcap"]
+    nopool = U.pooled(heads=1, kv_heads=1, dim=10, vdim=20, size=1000, pool=3, sink=True, v_mix=False)
+    del nopool["mixer"]["mask"]["pool"]
+    layers = [(U.latent(heads=1, dim=10, rot_dim=6, vdim=70, kv_rank=20, size=1, rot_dims=6), U.dense(ff=18)),
+              (plain, None),
+              (U.pooled(heads=2, kv_heads=2, dim=12, vdim=20, size=1, pool=1, sink=True), U.dense(ff=30)),
+              (U.pooled(heads=6, kv_heads=2, dim=20, vdim=20, size=3, pool=7, sink=False, v_mix=False), None),
+              (nopool, U.dense(ff=44)),
+              (U.capped(heads=6, kv_heads=2, dim=36, vdim=20, coef=1.5, every=1, softcap=2.0), U.dense(ff=25)),
+              (U.latent(heads=5, dim=12, rot_dim=4, vdim=12, kv_rank=100, size=1000, rot_dims=2, base=77.0, scale=0.4), None)]
+    cs = U.make_config(layers, width=100, vocab=77, eps=1e-6, logit_scale=1.0)
+    w = U.make_weights(cs, 5)
+    model = registry.load_model(U.save(str(tmp_path), cs, w), dt, DEV)
+    toks = tokens(48, cs[0]["vocab"], 6)
+    want = O.forward(toks, w, cs[0], F64)
+    b = batch_of(model)
+    got = [b.step([("a", toks[:29])], [list(range(29))])] + [b.step([("a", [t])]) for t in toks[29:]]
+    assert row_err(torch.cat(got), want) < TOL[dt]
+
+
+def test_wide_rows_and_wide_heads(tmp_path):
+    """Rows wider than 512 (the 16-byte norm kernel), heads of 136 | 72 and 128 + 64, a latent of 520 (the folded form's values go in two parts)."""
+    from llm_quest_amd import registry
+
+    layers = [(U.pooled(heads=2, kv_heads=1, dim=136, vdim=72, size=9, pool=4), U.dense(ff=64)),
+              (U.latent(heads=2, dim=128, rot_dim=64, vdim=24, kv_rank=520, size=17), None),
+              (U.capped(heads=2, kv_heads=1, dim=40, vdim=72), U.dense(ff=16))]
+    cs = U.make_config(layers, width=520, vocab=50)
+    w = U.make_weights(cs, 9)
+    toks = tokens(40, cs[0]["vocab"], 8)
+    want = O.forward(toks, w, cs[0], F64)
+    for dt in ("float32", "bfloat16"):
+        model = registry.load_model(U.save(str(tmp_path / dt), cs, w), dt, DEV)
+        b = batch_of(model)
+        got = [b.step([("a", toks[:21])], [list(range(21))])] + [b.step([("a", [t])]) for t in toks[21:]]
+        assert row_err(torch.cat(got), want) < TOL[dt]
+
+
+def test_greedy_generation_through_the_entry_point(models):
+    from llm_quest_amd.generate import generate_ragged
+
+    ms, cfg, w = models
+    prompts = [tokens(n, cfg["vocab"], 40 + n) for n in (4, 19, 9)]
+    out = generate_ragged(ms["float32"], prompts, max_gen=10)
+    for p, gen in zip(prompts, out):
+        assert len(gen) == 10
+        seq = list(p)
+        for t in gen:
+            lg = O.forward(seq, w, cfg, F64)[-1]
+            top = torch.topk(lg, 2)
+            if int(top.indices[0]) != t:
+                assert float(top.values[0] - top.values[1]) < 1e-4, "greedy token differs from the oracle's without a near tie"
+                break
+            seq.append(t)
+    first = out[1][2]
+    out2 = generate_ragged(ms["float32"], prompts, max_gen=10, eos_ids=[first])
+    assert out2[1] == out[1][: out[1].index(first)] and out2[0][: len(out2[0])] == out[0][: len(out2[0])]
+
+
+def test_trace_replay_program_end_to_end(checkpoint, tmp_path):
+    """bin/trace_run as a user runs it: a folder, steps on standard input (two prompts in one batch, then one token each, one request ending early and
+    its slot taken by a third), logits files out -- against the oracle."""
+    import json
+    import os
+    import subprocess
+    import sys
+
+    import numpy as np
+
+    folder, cfg, w = checkpoint
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    a, b, c = tokens(31, cfg["vocab"], 50), tokens(9, cfg["vocab"], 51), tokens(12, cfg["vocab"], 52)
+    steps = [{"step": 0, "entries": [{"id": "a", "tokens": a[:28], "want": [0, 13, 27]}, {"id": "b", "tokens": b[:8], "want": []}], "end": []},
+             {"step": 1, "entries": [{"id": "a", "tokens": a[28:29], "want": [0]}, {"id": "b", "tokens": b[8:9], "want": [0]}], "end": ["b"]},
+             {"step": 2, "entries": [{"id": "a", "tokens": a[29:30], "want": []}], "end": []},
+             {"step": 3, "entries": [{"id": "c", "tokens": c, "want": [11]}], "end": ["c"]},
+             {"step": 4, "entries": [{"id": "a", "tokens": a[30:31], "want": [0]}], "end": ["a"]}]
+    wa, wb, wc = oracle(cfg, w, a), oracle(cfg, w, b), oracle(cfg, w, c)
+    want = {0: torch.stack([wa[0], wa[13], wa[27]]), 1: torch.stack([wa[28], wb[8]]), 3: wc[11:12], 4: wa[30:31]}
+    for dt in ("float32", "bfloat16"):
+        out = tmp_path / dt
+        res = subprocess.run([sys.executable, os.path.join(root, "bin", "trace_run"), "--model", folder, "--dtype", dt, "--out", str(out), "--max-tokens", "64"],
+                             input="\n".join(json.dumps(s) for s in steps) + "\n", capture_output=True, text=True, timeout=300)
+        assert res.returncode == 0, res.stderr[-2000:]
+        assert [l for l in res.stdout.split("\n") if l.startswith("done")] == [f"done {i}" for i in range(5)]
+        assert not (out / "2.f32").exists()
+        for i, ref in want.items():
+            got = torch.from_numpy(np.fromfile(out / f"{i}.f32", dtype="<f4").reshape(-1, cfg["vocab"]))
+            assert got.shape == ref.shape and row_err(got, ref) < TOL[dt], (dt, i)
+
+
+# ------------------------------------------------------------------------------------------------------------------- mechanisms alone
+@pytest.mark.parametrize("width", [72, 100, 256, 520, 1000, 2048, 4100])
+def test_residual_sum_between_two_norms(width):
+    from llm_quest_amd import kernels_seq as S
+
+    g = torch.Generator().manual_seed(width)
+    T = 9
+    x, y = torch.randn(T, width, generator=g) * 3, torch.randn(T, width, generator=g) * 40
+    wp, wn = torch.rand(width, generator=g) + 0.5, torch.rand(width, generator=g) + 0.5
+    v = x.double() + O.rms_norm(y.double(), wp.double(), 1e-5)
+    for ydt in (F32, BF16):
+        yy = y.to(ydt)
+        v = x.double() + O.rms_norm(yy.double(), wp.double(), 1e-5)
+        x_out, h = S.sandwich_rmsnorm(x.to(DEV), 1e-5, y=yy.to(DEV), w_post=wp.to(DEV), w_next=wn.to(DEV), out_dtype=F32, x_out=True)
+        assert torch.allclose(x_out.cpu().double(), v, atol=2e-5) and row_err(h, O.rms_norm(v, wn.double(), 1e-5)) < 2e-6
+    # the output alone (the row is already summed), as bf16; the sum alone, written in place
+    _, hb = S.sandwich_rmsnorm(x.to(DEV), 1e-5, w_next=wn.to(DEV), out_dtype=BF16)
+    assert torch.equal(hb.cpu(), S.sandwich_rmsnorm(x.to(DEV), 1e-5, w_next=wn.to(DEV), out_dtype=F32)[1].cpu().to(BF16))
+    assert row_err(hb, O.rms_norm(x.double(), wn.double(), 1e-5)) < 5e-3
+    xd = x.to(DEV)
+    x_out, none = S.sandwich_rmsnorm(xd, 1e-5, y=y.to(DEV), w_post=wp.to(DEV), x_out=xd)
+    assert none is None and x_out is xd and torch.allclose(xd.cpu().double(), x.double() + O.rms_norm(y.double(), wp.double(), 1e-5), atol=2e-5)
+    # eps matters for a tiny sublayer output
+    tiny = y * 1e-4
+    _, h = S.sandwich_rmsnorm(x.to(DEV), 1e-5, y=tiny.to(DEV), w_post=wp.to(DEV), w_next=wn.to(DEV), out_dtype=F32)
+    assert row_err(h, O.rms_norm(x.double() + O.rms_norm(tiny.double(), wp.double(), 1e-5), wn.double(), 1e-5)) < 2e-6
+
+
+def test_xielu_and_the_sigmoid_gate_on_rows():
+    from llm_quest_amd import kernels_seq as S
+
+    g = torch.Generator().manual_seed(0)
+    for n in (70, 64):
+        z = torch.cat([torch.randn(5, n, generator=g) * 3, torch.tensor([[0.0, -1e-4, 1e-4, -30.0, 30.0] + [0.5] * (n - 5)])])
+        for p, q in ((0.3, -0.7), (-2.0, 1.5), (25.0, 0.0)):
+            par = torch.tensor([p, q])
+            got = S.act_rows(z.to(DEV), S.ACT_XIELU, params=par.to(DEV))
+            assert row_err(got, O.xielu(z.double(), par[0].double(), par[1].double())) < 2e-6
+        wide = torch.randn(6, 3 * n, generator=g).to(DEV)  # rows that are views with a pitch of their own
+        got = S.act_rows(wide[:, :n], S.ACT_SIGMOID_GATE, gate=wide[:, n : 2 * n], out_dtype=BF16)
+        want = wide[:, :n].double() * torch.sigmoid(wide[:, n : 2 * n].double())
+        assert row_err(got, want) < 5e-3
+        assert row_err(S.act_rows(wide[:, 1 : n + 1], S.ACT_SIGMOID_GATE, gate=wide[:, n : 2 * n]), wide[:, 1 : n + 1].double() * torch.sigmoid(wide[:, n : 2 * n].double())) < 2e-6
+
+
+def test_latent_rows_in_the_rotate_half_layout():
+    from llm_quest_amd import kernels_seq as S
+
+    g = torch.Generator().manual_seed(4)
+    R, dr, dims, base = 20, 10, 6, 1e4
+    pos = [0, 1, 2, 63, 64, 1000]
+    src = torch.randn(len(pos), R + dr, generator=g)
+    w = torch.rand(R, generator=g) + 0.5
+    full = torch.zeros(pos[-1] + 1, 1, dr, dtype=F64)
+    full[pos, 0] = src[:, R:].double()
+    want = torch.cat([O.rms_norm(src[:, :R].double(), w.double(), 1e-5), O.rotary_half(full, dims, base)[pos, 0]], dim=1)
+    cache = torch.zeros(40, R + dr, device=DEV)
+    rows = [7, 3, 11, 0, 39, 20]
+    S.latent_kv_append(src.to(DEV), R, dr, w.to(DEV), 1e-5, dev_i32(pos), dev_i32(rows), S.rope_frequencies(dims, base, DEV), dims, cache, layout=1)
+    assert row_err(cache[rows], want) < 1e-5
+    assert float(cache[[1, 2, 4, 5, 6]].abs().max()) == 0.0
+
+
+def test_query_temperature_and_value_mixing_in_the_row_kernel():
+    """Positions just before, at and just after the steps of the temperature (p + 1 a multiple of `every`)."""
+    from llm_quest_amd import kernels_seq as S
+
+    g = torch.Generator().manual_seed(5)
+    H, G, d, dv, every, coef, lam = 3, 1, 10, 6, 7, 0.9, 0.3
+    pos = [0, 5, 6, 7, 12, 13, 14, 699, 700]
+    src = torch.randn(len(pos), (H + G) * d + G * dv, generator=g)
+    mix = torch.randn(len(pos), G * dv + 3, generator=g)
+    cache = torch.zeros(len(pos), G * (d + dv), device=DEV)
+    mixd = mix.to(DEV)
+    q = S.qkv_rows_append(src.to(DEV), H, G, d, dv, None, None, None, 1e-5, None, 0, 0, None, dev_i32(pos), dev_i32(list(range(len(pos)))), cache, q_temp=(coef, every),
+                          vmix=mixd[:, 1 : 1 + G * dv], lam=lam)
+    temp = torch.tensor([1.0 + coef * torch.log(torch.tensor(float((p + 1) // every + 1), dtype=F64)) for p in pos], dtype=F64)
+    full = O.query_temperature(pos[-1] + 1, coef, every, F64)
+    assert torch.allclose(full[pos], temp)
+    assert row_err(q, src[:, : H * d].double() * temp[:, None]) < 2e-6
+    assert row_err(cache[:, : G * d], src[:, H * d : (H + G) * d].double()) < 1e-7
+    assert row_err(cache[:, G * d :], O.mix_values(src[:, (H + G) * d :].double(), mix[:, 1 : 1 + G * dv].double(), lam)) < 2e-6
+
+
+def _attention_alone(dt, H, G, d, dv, size, pool, sink, cap, portions, hot, seed=0, slots=(0,), window_attr=None):
+    """``SlidingWindowAttention`` alone with identity projections: the module's input rows ARE [q | k | v], its output's first H * dv entries the attention's.
+    ``portions``: per step the new tokens of every sequence ([[n of sequence 0, n of sequence 1, ...], ...], 0 = the sequence pauses).  ``hot``: keys made to match
+    later queries with a large value.  Returns per sequence (got, want)."""
+    from llm_quest_amd.common.mixers import SeqStep, SlidingWindowAttention
+    from llm_quest_amd.utils import SlotStateCache
+
+    act = F32 if dt == "float32" else BF16
+    n_in = (H + G) * d + G * dv
+    width = max(n_in, H * dv)
+    mod = SlidingWindowAttention(width, H, G, d, dv, d ** -0.5, size, 0, 0, 1e4, 1e-5, 0, qk_norm=False, bias=False, temp=False, softcap=cap, pool=pool, sink=sink is not None)
+    mod.w_qkv.data.copy_(torch.eye(n_in, width))
+    mod.w_o.data.copy_(torch.eye(width, H * dv))
+    if sink is not None:
+        mod.sink.data.copy_(sink)
+    mod = mod.to(DEV)
+    n_seq = len(portions[0])
+    totals = [sum(p[i] for p in portions) for i in range(n_seq)]
+    g = torch.Generator().manual_seed(seed)
+    data = []
+    for T in totals:
+        q, k, v = torch.randn(T, H, d, generator=g) * 2, torch.randn(T, G, d, generator=g), torch.randn(T, G, dv, generator=g)
+        for j in hot:
+            if j < T:
+                i = min(T - 1, j + (size or 3) + pool)
+                k[j, :] = q[i, 0] * 1.5
+                v[j, :] = 20.0 + j
+        rows = torch.cat([q.reshape(T, -1), k.reshape(T, -1), v.reshape(T, -1), torch.zeros(T, width - n_in)], dim=1).to(act)
+        data.append(rows)
+    cache = SlotStateCache([mod.cache_spec()], 1 << 16, DEV, act, slots=max(slots) + 1)
+    cache.initial_chunk_size, cache.chunk_size = 8, 16
+    at, got = [0] * n_seq, [[] for _ in range(n_seq)]
+    for step in portions:
+        live = [i for i in range(n_seq) if step[i]]
+        st = SeqStep(cache, [(slots[i], [0] * step[i]) for i in live], DEV, act)
+        h = torch.cat([data[i][at[i] : at[i] + step[i]] for i in live]).to(DEV)
+        out = mod.step(h, st, out_dtype=F32)
+        o = 0
+        for i in live:
+            got[i].append(out[o : o + step[i], : H * dv])
+            o += step[i]
+            at[i] += step[i]
+            cache.advance(slots[i], [0] * step[i])
+    res = []
+    for i, T in enumerate(totals):
+        r = data[i].double()
+        q, k, v = r[:, : H * d].reshape(T, H, d), r[:, H * d : (H + G) * d].reshape(T, G, d), r[:, (H + G) * d : n_in].reshape(T, G, dv)
+        kp, vp = (k.to(act).double(), v.to(act).double())
+        if pool and act == BF16:  # the pooled rows are stored in the cache's dtype
+            extra = lambda i_, k=kp, v=vp: tuple(t.to(BF16).double() for t in O.pooled_blocks(k, v, i_, size, pool))
+        else:
+            extra = (lambda i_, k=kp, v=vp: O.pooled_blocks(k, v, i_, size, pool)) if pool else None
+        want = O.softmax_attention(q, kp, vp, d ** -0.5, lambda i_: O.window_keys(i_, size), cap=cap or None, sink=None if sink is None else sink.double(), extra=extra)
+        res.append((torch.cat(got[i]), want.reshape(T, H * dv)))
+    return res
+
+
+ATT_TOL = {"float32": 5e-5, "bfloat16": 3e-2}
+
+
+@pytest.mark.parametrize("dt", ["float32", "bfloat16"])
+@pytest.mark.parametrize("size,pool", [(13, 5), (16, 8), (1, 1), (3, 7), (70, 4)])
+def test_window_with_pooled_blocks_in_prompts_and_decoding(dt, size, pool):
+    """Every query of a 200-token sequence against the oracle, with hot keys every few positions: a key that is one position too long or too short in the
+    window, or a block that is seen one token early or late, changes some row by far more than the tolerance.  The prompt crosses the kernels' 64-key and
+    32- / 128-query steps; the decoded tokens then move every edge one position at a time."""
+    hot = list(range(2, 200, 7))
+    sink = torch.tensor([0.5, -1.0, 2.0, 0.0])
+    (got, want), = _attention_alone(dt, 4, 2, 24, 40, size, pool, sink, 0.0, [[150]] + [[1]] * 50, hot)
+    assert row_err(got, want) < ATT_TOL[dt]
+    assert float(want.abs().max()) > 15  # the hot keys do come through
+
+
+@pytest.mark.parametrize("dt", ["float32", "bfloat16"])
+def test_pooled_blocks_over_portions_and_two_sequences(dt):
+    """Two sequences in different slots advance by unequal portions (1, 2, several; one pauses): blocks are completed by different steps, several in one step
+    or none, and a portion starts in the middle of a block."""
+    portions = [[37, 5], [1, 2], [2, 1], [9, 0], [0, 30], [1, 1], [26, 3], [1, 1], [2, 2], [33, 64]]
+    res = _attention_alone(dt, 6, 2, 16, 24, 11, 4, torch.tensor([1.0, 0.0, -2.0, 0.3, 0.3, 3.0]), 0.0, portions, list(range(1, 110, 5)), seed=3, slots=(2, 0))
+    for got, want in res:
+        assert row_err(got, want) < ATT_TOL[dt]
+
+
+@pytest.mark.parametrize("dt", ["float32", "bfloat16"])
+def test_sink_alone_changes_only_the_denominator(dt):
+    """No window, no pool: with a large sink the outputs shrink by the sink's share; one-token steps over 700 cached keys deal the keys to several workgroups
+    in bf16, whose joined result must still count the sink once."""
+    sink = torch.tensor([4.0, -3.0])
+    (got, want), = _attention_alone(dt, 2, 1, 32, 48, 0, 0, sink, 0.0, [[700]] + [[1]] * 3, [5, 650], seed=1)
+    assert row_err(got, want) < ATT_TOL[dt]
+    (plain, want0), = _attention_alone(dt, 2, 1, 32, 48, 0, 0, None, 0.0, [[700]] + [[1]] * 3, [5, 650], seed=1)
+    assert row_err(plain, want0) < ATT_TOL[dt]
+    # the first query sees one key: its weight is 1 without a sink and 1 / (1 + exp(sink - score)) with it
+    assert float((plain[0] - got[0]).abs().max()) > 0.05 * float(plain[0].abs().max())
+
+
+@pytest.mark.parametrize("dt", ["float32", "bfloat16"])
+@pytest.mark.parametrize("cap", [1.5, 24.0])
+def test_capped_scores_see_every_earlier_key(dt, cap):
+    """Scores far above the cap saturate: a hot key at the very start still shares the weight with the other hot keys instead of taking it all."""
+    (got, want), = _attention_alone(dt, 4, 4, 24, 24, 0, 0, None, cap, [[130]] + [[1]] * 5, [0, 64, 100], seed=2)
+    assert row_err(got, want) < ATT_TOL[dt]
+
+
+@pytest.mark.parametrize("dt", ["float32", "bfloat16"])
+def test_latent_attention_window_edges_prompt_and_folded_form(dt):
+    """The mixer alone with random weights against the oracle over a prompt and then token by token (the folded form reads the cache rows as keys and values of
+    every head): windows of 1, 5 and 64 keys; a rotation of part of the rotated entries."""
+    from llm_quest_amd.common.mixers import LatentAttention, SeqStep
+    from llm_quest_amd.utils import SlotStateCache
+
+    act = F32 if dt == "float32" else BF16
+    for size, H, dn, dr, dv, R, dims in ((1, 2, 8, 4, 8, 16, 4), (5, 3, 24, 16, 40, 48, 12), (64, 4, 32, 8, 16, 64, 8)):
+        width = 72
+        layer = U.latent(heads=H, dim=dn, rot_dim=dr, vdim=dv, kv_rank=R, size=size, rot_dims=dims)
+        cs = U.make_config([(layer, None)], width=width)
+        w = U.make_weights(cs, size)
+        m = layer["mixer"]
+        mod = LatentAttention(width, H, dn, dr, dv, 0, R, m["scale"], dims, m["rot"]["base"], 1e-5, 0, rot_layout=1, window=size, gate=True)
+        p = "l0.mix."
+        mod.w_down.data.copy_(torch.cat([w[p + "q"], w[p + "dkv"], w[p + "g"]]))
+        mod.kv_norm.data.copy_(w[p + "dkv.norm"])
+        mod.w_ukv.data.copy_(torch.cat([w[p + "uk"], w[p + "uv"]]))
+        mod.w_o.data.copy_(w[p + "o"])
+        mod = mod.to(DEV)
+        T = 150
+        h = (torch.randn(T, width, generator=torch.Generator().manual_seed(size)) * 1.5).to(act)
+        want = O.latent_attention_mixer(h.double(), {k: v.double() for k, v in w.items()}, p, m, 1e-5, {})
+        cache = SlotStateCache([mod.cache_spec()], 1 << 16, DEV, act, slots=1)
+        got = []
+        for n in [100] + [1] * 50:
+            st = SeqStep(cache, [(0, [0] * n)], DEV, act)
+            at = cache.length[0]
+            got.append(mod.step(h[at : at + n].to(DEV), st, out_dtype=F32))
+            cache.advance(0, [0] * n)
+        assert row_err(torch.cat(got), want) < (2e-5 if dt == "float32" else 3e-2), (size, H)
+
+
+@pytest.mark.parametrize("dt", ["float32", "bfloat16"])
+@pytest.mark.parametrize("size,pool", [(300, 16), (257, 0)])
+def test_one_token_steps_deal_a_long_windows_keys_to_several_workgroups(dt, size, pool):
+    """900 cached keys under a window of some 300: the bf16 kernel deals the window's range (which starts in the middle of a 64-key step) to several workgroups,
+    the first of which also takes the pooled rows; hot keys sit at both edges of the window of the decoded tokens."""
+    hot = [899 - size, 900 - size, 901 - size, 902 - size, 640, 898, 3, 40]
+    (got, want), = _attention_alone(dt, 4, 2, 32, 48, size, pool, torch.tensor([0.5, -1.0, 2.0, 0.0]), 0.0, [[900]] + [[1]] * 4, hot, seed=7)
+    assert row_err(got[900:], want[900:]) < ATT_TOL[dt] and row_err(got, want) < ATT_TOL[dt]
