@@ -268,9 +268,11 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(LatAttnArgs p, in
     }
     int n_keys = past + min(tok0 + tm, n_new);
     int key_lo = 0;
-    if (p.splits > 1) {  // this workgroup's share: whole 64-key steps
-        const int span = ((n_keys + MKT - 1) / MKT + p.splits - 1) / p.splits * MKT;
-        key_lo = split * span;
+    const int win_lo = p.window > 0 ? past + tok0 - p.window + 1 : 0;  // keys below it are outside the window of every row of the tile
+    if (p.splits > 1) {  // this workgroup's share: whole 64-key steps of the range the tile can see (under a plain window that range starts at its lower edge)
+        const int lo0 = (p.window > 0 && p.keep_first == 0 && win_lo > 0) ? win_lo / MKT * MKT : 0;
+        const int span = ((n_keys - lo0 + MKT - 1) / MKT + p.splits - 1) / p.splits * MKT;
+        key_lo = lo0 + split * span;
         n_keys = min(n_keys, key_lo + span);
     }
     // the last key any row of this WAVE may see (its rows are consecutive, so its last valid row has the largest limit)
@@ -287,7 +289,6 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(LatAttnArgs p, in
     const float sc2 = p.scale * 1.4426950408889634f;
 
     const int kvh = head0 / p.kv_rep;
-    const int win_lo = p.window > 0 ? past + tok0 - p.window + 1 : 0;
     // pooled rows any row of the tile may see (a tile's first key share takes them), and those this lane's query sees
     const int n_pool = (p.pool > 0 && split == 0) ? pooled_visible(past + min(tok0 + tm, n_new) - 1, p.window, p.pool) : 0;
     const int pool_steps = (n_pool + MKT - 1) / MKT;

@@ -199,7 +199,61 @@ extern "C" int mi355_pool_rows_update(int n_seq, int max_blocks, int width, int 
 // kind 0 (xIELU, params = two raw numbers p, q):  z > 0: softplus(p) z^2 + z / 2;  z <= 0: (1/2 + softplus(q)) (exp(z) - 1 - z) + z / 2.
 // kind 1 (sigmoid gate): out = x * sigmoid(gate), gate rows of their own dtype and pitch.
 __device__ __forceinline__ float softplus_f(float a) { return a > 20.f ? a : log1pf(expf(a)); }
-__device__ __forceinline__ float xielu_f(float z, float ap, float aq) { return z > 0.f ? ap * z * z + 0.5f * z : aq * (expm1f(z) - z) + 0.5f * z; }
+// exp(z) - 1 - z for z <= 0 without cancellation: the series z^2 (1/2! + z/3! + ... + z^8/10!) down to -1/2, the exponential itself below
+__device__ __forceinline__ float exp_minus_1_minus_z(float z) {
+    if (z < -0.5f) return expf(z) - 1.0f - z;
+    float s = 1.0f / 3628800.0f;
+    s = fmaf(s, z, 1.0f / 362880.0f);
+    s = fmaf(s, z, 1.0f / 40320.0f);
+    s = fmaf(s, z, 1.0f / 5040.0f);
+    s = fmaf(s, z, 1.0f / 720.0f);
+    s = fmaf(s, z, 1.0f / 120.0f);
+    s = fmaf(s, z, 1.0f / 24.0f);
+    s = fmaf(s, z, 1.0f / 6.0f);
+    s = fmaf(s, z, 0.5f);
+    return z * z * s;
+}
+__device__ __forceinline__ float xielu_f(float z, float ap, float aq) { return z > 0.f ? ap * z * z + 0.5f * z : aq * exp_minus_1_minus_z(z) + 0.5f * z; }
+// eight consecutive bf16 (16-byte aligned) <-> floats
+__device__ __forceinline__ void ld8_bf(const void* p, int64_t i, float* v) {
+    const u32x4 r = *(const u32x4*)((const bf16_t*)p + i);
+#pragma unroll
+    for (int q = 0; q < 4; ++q) v[2 * q] = __uint_as_float(r[q] << 16), v[2 * q + 1] = __uint_as_float(r[q] & 0xffff0000u);
+}
+__device__ __forceinline__ void st8_bf(void* p, int64_t i, const float* v) {
+    *(u32x4*)((bf16_t*)p + i) = u32x4{pack_bf2(v[0], v[1]), pack_bf2(v[2], v[3]), pack_bf2(v[4], v[5]), pack_bf2(v[6], v[7])};
+}
+
+// bf16 rows in and out, eight entries per thread (16-byte accesses); the gate may be bf16 or fp32
+__global__ __launch_bounds__(256) void act_rows_bf8_kernel(int64_t R, int n, const void* __restrict__ x, int64_t ldx, const void* __restrict__ gate, int g_dt, int64_t ldg, int kind,
+                                                           const float* __restrict__ params, void* __restrict__ out, int64_t ldo) {
+    float ap = 0.f, aq = 0.f;
+    if (kind == 0) ap = softplus_f(params[0]), aq = 0.5f + softplus_f(params[1]);
+    const int nw = n / 8;
+    const int64_t total = R * nw;
+    for (int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; e < total; e += (int64_t)gridDim.x * blockDim.x) {
+        const int64_t r = e / nw;
+        const int i = 8 * (int)(e % nw);
+        float a[8], o[8];
+        ld8_bf(x, r * ldx + i, a);
+        if (kind == 0) {
+#pragma unroll
+            for (int q = 0; q < 8; ++q) o[q] = xielu_f(a[q], ap, aq);
+        } else {
+            float g[8];
+            if (g_dt == MI355_DT_F32) {
+                const f32x4 g0 = *(const f32x4*)((const float*)gate + r * ldg + i), g1 = *(const f32x4*)((const float*)gate + r * ldg + i + 4);
+#pragma unroll
+                for (int q = 0; q < 4; ++q) g[q] = g0[q], g[4 + q] = g1[q];
+            } else {
+                ld8_bf(gate, r * ldg + i, g);
+            }
+#pragma unroll
+            for (int q = 0; q < 8; ++q) o[q] = a[q] / (1.0f + expf(-g[q]));
+        }
+        st8_bf(out, r * ldo + i, o);
+    }
+}
 
 template <bool VEC>
 __global__ __launch_bounds__(256) void act_rows_kernel(int64_t R, int n, const void* __restrict__ x, int x_dt, int64_t ldx, const void* __restrict__ gate, int g_dt, int64_t ldg,
@@ -235,6 +289,12 @@ extern "C" int mi355_act_rows(int64_t rows, int n, const void* x, int x_dt, int6
                               void* out, int out_dt, int64_t ldo, void* stream) {
     MI355_REQUIRE(rows > 0 && n > 0 && x && out && sand_dt_ok(x_dt) && sand_dt_ok(out_dt) && ldx >= n && ldo >= n && (kind == 0 || kind == 1), "act_rows: bad arguments");
     MI355_REQUIRE(kind == 0 ? params != nullptr : (gate && sand_dt_ok(g_dt) && ldg >= n), "act_rows: xIELU needs its two numbers, a gate its rows");
+    if (x_dt == MI355_DT_BF16 && out_dt == MI355_DT_BF16 && n % 8 == 0 && ldx % 8 == 0 && ldo % 8 == 0 && sand_al16(x) && sand_al16(out) &&
+        (kind == 0 || (ldg % 8 == 0 && sand_al16(gate)))) {
+        act_rows_bf8_kernel<<<sand_grid(rows * (n / 8), 256, 65535 * 8), 256, 0, ST(stream)>>>(rows, n, x, ldx, gate, g_dt, ldg, kind, params, out, ldo);
+        MI355_LAUNCH_CHECK("act_rows");
+        return 0;
+    }
     const bool vec = n % 4 == 0 && ldx % 4 == 0 && ldo % 4 == 0 && sand_al16(x) && sand_al16(out) && (kind == 0 || (ldg % 4 == 0 && sand_al16(gate)));
     const int64_t total = rows * (vec ? n / 4 : n);
     const int g = sand_grid(total, 256, 65535 * 8);

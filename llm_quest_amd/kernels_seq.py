@@ -236,13 +236,13 @@ def linear(x, w, out_dtype=None, bias=None):
     return bgemm(x, w, out, M, N, Kd, bias=bias)
 
 
-def attn_key_splits(n_seq, head_tiles, max_new, hm, max_keys):
+def attn_key_splits(n_seq, head_tiles, max_new, hm, max_keys, per_split=256):
     """Workgroups per tile of the MFMA attention: a step with few query tiles and long caches (one-token steps) deals each tile's keys to several, about
-    256 keys each, as many as fill the chip's 256 CUs once."""
+    ``per_split`` keys each, as many as fill the chip's 256 CUs once."""
     tiles = n_seq * head_tiles * -(-max_new * hm // 128)
-    if max_keys <= 512 or tiles >= 128:
+    if max_keys <= 2 * per_split or tiles >= 128:
         return 1
-    return max(1, min(-(-max_keys // 256), 32, 256 // tiles))
+    return max(1, min(-(-max_keys // per_split), 32, 256 // tiles))
 
 
 def latent_attn(q, k1, k2, v, out, H, hm, D1, D2, DV, q_hs, k1_hs, v_hs, o_hs, desc, max_new, scale, max_keys=0, kv_rep=1, window=0, keep_first=0, softcap=0.0,
@@ -274,10 +274,13 @@ def latent_attn(q, k1, k2, v, out, H, hm, D1, D2, DV, q_hs, k1_hs, v_hs, o_hs, d
         _i32(t, "latent_attn(desc)", n_seq)
     mfma = v.dtype == BF16
     splits, ws = 1, None
-    # (a window that can hide keys leaves a one-token step window + keep_first visible keys, and the kernel skips the others 64 at a time: nothing to deal out)
-    if mfma and D1 + D2 <= 320 and DV <= 256 and max_keys and (not window or window >= max_keys):
+    # A plain window leaves a tile window + its own tokens to see: that range is dealt out, in finer shares (a one-token step over it is a chain of
+    # dependent 64-key steps in very few workgroups).  A window that also keeps the first tokens is not dealt out: the kernel skips what lies between.
+    plain_window = window and window < max_keys and not keep_first
+    if mfma and D1 + D2 <= 320 and DV <= 256 and max_keys and (not window or window >= max_keys or plain_window):
         head_tiles = -(-H // hm)
-        splits = attn_key_splits(n_seq, head_tiles, max_new, hm, max_keys)
+        tile_tokens = min(max_new, -(-128 // hm))
+        splits = attn_key_splits(n_seq, head_tiles, max_new, hm, min(max_keys, window + tile_tokens - 1), 128) if plain_window else attn_key_splits(n_seq, head_tiles, max_new, hm, max_keys)
         if splits > 1:
             dvp = 32 if DV <= 32 else 64 if DV <= 64 else 128 if DV <= 128 else 256
             ws = torch.empty(n_seq * head_tiles * -(-max_new * hm // 128) * splits * 128 * (2 + dvp), dtype=F32, device=v.device)

@@ -1,6 +1,8 @@
 """Serving throughput of the registry models with random weights: prompts (one packed step) and one-token steps through the slot cache, beside the
 closest existing model of the package at equal width and depth -- the Qwen3.5 hybrid text stack (gated delta net + gated attention, dense SwiGLU) through
 its own cache.  ``bench.py --serve gemepel`` (or ``--serve mepatar``) prints the result as one JSON line; the default workload of ``bench.py`` is untouched.
+``--serve mopalorn`` stands beside a Mepatar stack of sliding-window attention layers with dense feed-forwards at equal width, depth, heads and parameter
+count: the package's closest model to an all-attention decoder with dense layers.
 
 Sizes resemble real layers (random weights; what is generated means nothing): width 1024 / 2048, 4 layers (three linear-attention layers and one softmax-
 attention layer, as the Qwen3.5 stack has them), 16 experts of which 2 run per token."""
@@ -72,6 +74,58 @@ def random_mepatar(width, heads, device):
         elif name.endswith("A_log"):
             p.data.fill_(-2.0)
     return model
+
+
+def mopalorn_config(width, heads, vocab=32000):
+    """Four layers, one of each kind and a second latent one: windowed attention with pooled blocks and a sink (512 keys + one row per 32 older tokens), latent
+    attention (128 + 64 | 128 per head, latent 256, 512-key window, gated), capped attention over all keys with a query temperature, latent attention again;
+    grouped queries over 2 key heads; every layer with a dense xIELU feed-forward of ff = 4 width; values mixed from the first layer on."""
+    gqa = {"heads": heads, "kv_heads": 2, "dim": 128, "vdim": 128, "scale": 128 ** -0.5, "v_mix": True}
+    lat = {"heads": heads, "dim": 128, "rot_dim": 64, "vdim": 128, "kv_rank": 256, "mask": {"size": 512}, "rot": {"dims": 64, "base": 1e6}, "scale": 192 ** -0.5}
+    mlp = {"kind": "dense", "ff": 4 * width}
+    layers = [{"type": "attention_2", "mixer": dict(gqa, mask={"size": 512, "pool": 32}), "mlp": mlp}, {"type": "latent_attention", "mixer": lat, "mlp": mlp},
+              {"type": "attention", "mixer": dict(gqa, q_temp={"coef": 0.25, "every": 128}, softcap=50.0), "mlp": mlp}, {"type": "latent_attention", "mixer": lat, "mlp": mlp}]
+    return {"architecture": "Mopalorn", "vocab": vocab, "width": width, "norm": {"eps": 1e-6}, "logit_scale": 0.125, "layers": layers}
+
+
+def _fill_random(model, device):
+    g = torch.Generator(device=device).manual_seed(7)
+    for name, p in model.named_parameters():
+        if p.dim() >= 2:
+            p.data.copy_((torch.randn(p.shape, device=device, generator=g) / p.shape[-1] ** 0.5).to(BF16))
+        elif "norm" in name or name.endswith("temp"):
+            p.data.fill_(1.0)
+        elif name.endswith("lam") or name.endswith("act"):
+            p.data.fill_(0.25)
+    return model
+
+
+def random_mopalorn(width, heads, device):
+    from llm_quest_amd.mopalorn.mopalorn_model import MopalornConfig, MopalornModel
+
+    with torch.device(device):
+        model = MopalornModel(MopalornConfig(mopalorn_config(width, heads)))
+    return _fill_random(model, device)
+
+
+def mepatar_attention_config(width, heads, vocab=32000):
+    """The reference beside Mopalorn: four Mepatar layers of sliding-window attention (512 keys + 4 kept, grouped queries over 2 key heads, 128 | 128) with
+    the dense gated feed-forward at ff = 8/3 width (as many weights as an un-gated layer of 4 width), no input convolution, norms in one group."""
+    att = {"heads": heads, "kv_heads": 2, "dim": 128, "vdim": 128, "mask": {"size": 512, "keep_first": 4}, "rot": {"dims": 64, "base": 1e6}, "scale": 128 ** -0.5}
+    layers = [{"type": "attention", "mixer": att, "mlp": {"kind": "dense", "ff": (8 * width // 3 + 63) // 64 * 64}} for _ in range(4)]
+    return {"architecture": "Mepatar", "vocab": vocab, "width": width, "norm": {"eps": 1e-6, "groups": 1}, "canon": {"taps": 1}, "embedding": {"scale": 1.0}, "layers": layers}
+
+
+def bench_mopalorn(width, heads, batch, prompt, steps, warmup, device):
+    return bench_ragged(random_mopalorn(width, heads, device), f"mopalorn-w{width}", batch, prompt, steps, warmup)
+
+
+def bench_mepatar_attention(width, heads, batch, prompt, steps, warmup, device):
+    from llm_quest_amd.mepatar.mepatar_model import MepatarConfig, MepatarModel
+
+    with torch.device(device):
+        model = MepatarModel(MepatarConfig(mepatar_attention_config(width, heads)))
+    return bench_ragged(_fill_random(model, device), f"mepatar-attention-w{width}", batch, prompt, steps, warmup)
 
 
 def _time(fn, warmup, steps):
@@ -172,14 +226,15 @@ def bench_qwen35(width, heads, batch, prompt, steps, warmup, device):
 
 
 def run(which, steps, warmup, sizes=((1024, 8), (2048, 16)), batch=8, prompt=1024, device="cuda", with_reference=True):
-    benches = {"gemepel": bench_gemepel, "mepatar": bench_mepatar}
+    benches = {"gemepel": bench_gemepel, "mepatar": bench_mepatar, "mopalorn": bench_mopalorn, "mepatar-attention": bench_mepatar_attention}
     if which not in benches:
         raise SystemExit(f"--serve: unknown model {which!r} (known: {sorted(benches)})")
+    reference = bench_mepatar_attention if which == "mopalorn" else bench_qwen35
     rows = []
     for width, heads in sizes:
         rows.append(benches[which](width, heads, batch, prompt, steps, warmup, device))
         if with_reference:
-            rows.append(bench_qwen35(width, heads, batch, prompt, steps, warmup, device))
+            rows.append(reference(width, heads, batch, prompt, steps, warmup, device))
     out = {"metric": "serving throughput (random weights)", "unit": "tokens/s", "batch": batch, "prompt": prompt, "steps": steps, "warmup": warmup,
            "dtype": "bf16", "data": "synthetic", "rows": rows}
     print(json.dumps(out))
