@@ -123,3 +123,18 @@ def test_slot_cache_keeps_pooled_rows_through_growth():
     assert c.capacity >= 30 and c.pool_capacity(0) == -(-c.capacity // 4) and c.slots == 2
     assert float(c.pooled[0][a, 2, 0]) == 7.0 and float(c.rows[0][a, 9, 0]) == 5.0 and float(c.pooled[0][b].abs().max()) == 0.0
     assert c.pooled2d(0).shape == (2 * c.pool_capacity(0), 6)
+
+
+def test_bench_configurations_parse():
+    """The serving bench's Mopalorn model and its reference stack are valid configurations of their designs with equal layer weights (to 1 %)."""
+    from llm_quest_amd import serve_bench as B
+    from llm_quest_amd.mepatar.mepatar_model import MepatarConfig
+    from llm_quest_amd.mopalorn.mopalorn_model import MopalornConfig
+
+    for width, heads in ((1024, 8), (2048, 16)):
+        c = MopalornConfig(B.mopalorn_config(width, heads))
+        assert c.v_mix == ["first", None, "mix", None] and len(c.layers) == 4
+        r = MepatarConfig(B.mepatar_attention_config(width, heads))
+        ff_new = sum(2 * width * l["mlp"]["ff"] for l in c.layers)
+        ff_ref = sum(3 * width * l["mlp"]["ff"] for l in r.layers)
+        assert abs(ff_new - ff_ref) < 0.01 * ff_new
