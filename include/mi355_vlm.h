@@ -562,7 +562,8 @@ int mi355_bgemm(int batch, int M, int N, int K, const void* A, int a_dt, int64_t
  * key j of it is K1 row k1_row0[s] + j (head stride k1_hs, D1 wide), K2 row k2_row0[s] + j (shared by heads, D2 wide), value row v_row0[s] + j.
  * Q fp32 [.., H, D1 + D2]; K1 / K2 / V / O of dtype dt.  A tile covers 32 / hm tokens x hm heads (hm > 1 needs k1_hs == v_hs == 0); the MFMA path (bf16,
  * D1 + D2 <= 320, DV <= 256) 128 / hm tokens, and with splits > 1 deals a tile's keys to that many workgroups whose partial results meet in ws
- * (n_seq * head tiles * token tiles * splits * 128 * (2 + DV rounded up to 32 / 64 / 128 / 256) floats).
+ * (n_seq * head tiles * token tiles * splits * 128 * (2 + DV rounded up to 32 / 64 / 128 / 256) floats).  Under a plain window (keep_first == 0) the shares start
+ * at the window's lower edge, and pooled rows (below) are part of what is dealt out.
  * Grouped queries: head h reads key / value head h / kv_rep (strides k1_hs / v_hs per key / value head; hm may then divide kv_rep).  window > 0: the query
  * at position i sees key j <= i only if i - j < window or j < keep_first (a sliding window that keeps the first tokens); window 0: every j <= i.
  * softcap > 0: score <- softcap * tanh(score / softcap) after the scale.  sink (fp32 [H], may be NULL): exp(sink[h]) joins head h's softmax denominator.

@@ -266,14 +266,19 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(LatAttnArgs p, in
             qf[st] = __builtin_bit_cast(bf16x4, pk);
         }
     }
-    int n_keys = past + min(tok0 + tm, n_new);
-    int key_lo = 0;
+    const int n_keys = past + min(tok0 + tm, n_new);
     const int win_lo = p.window > 0 ? past + tok0 - p.window + 1 : 0;  // keys below it are outside the window of every row of the tile
-    if (p.splits > 1) {  // this workgroup's share: whole 64-key steps of the range the tile can see (under a plain window that range starts at its lower edge)
-        const int lo0 = (p.window > 0 && p.keep_first == 0 && win_lo > 0) ? win_lo / MKT * MKT : 0;
-        const int span = ((n_keys - lo0 + MKT - 1) / MKT + p.splits - 1) / p.splits * MKT;
-        key_lo = lo0 + split * span;
-        n_keys = min(n_keys, key_lo + span);
+    // The tile's work is a list of 64-row steps: first the pooled rows any of its rows may see, then the keys from key_lo on (under a plain window dealt
+    // out to several workgroups that is the window's lower edge, else 0: steps below a window are skipped one by one).  Workgroup `split` takes its share.
+    const int n_pool = p.pool > 0 ? pooled_visible(n_keys - 1, p.window, p.pool) : 0;
+    const int pool_steps = (n_pool + MKT - 1) / MKT;
+    const int key_lo = (p.splits > 1 && p.window > 0 && p.keep_first == 0 && win_lo > 0) ? win_lo / MKT * MKT : 0;
+    const int all_steps = pool_steps + (n_keys - key_lo + MKT - 1) / MKT;
+    int v_lo = 0, v_hi = all_steps;
+    if (p.splits > 1) {
+        const int per = (all_steps + p.splits - 1) / p.splits;
+        v_lo = split * per;
+        v_hi = min(all_steps, v_lo + per);
     }
     // the last key any row of this WAVE may see (its rows are consecutive, so its last valid row has the largest limit)
     int wave_lim = lim;
@@ -289,20 +294,14 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(LatAttnArgs p, in
     const float sc2 = p.scale * 1.4426950408889634f;
 
     const int kvh = head0 / p.kv_rep;
-    // pooled rows any row of the tile may see (a tile's first key share takes them), and those this lane's query sees
-    const int n_pool = (p.pool > 0 && split == 0) ? pooled_visible(past + min(tok0 + tm, n_new) - 1, p.window, p.pool) : 0;
-    const int pool_steps = (n_pool + MKT - 1) / MKT;
-    const int npv = p.pool > 0 ? pooled_visible(lim, p.window, p.pool) : 0;
+    const int npv = p.pool > 0 ? pooled_visible(lim, p.window, p.pool) : 0;  // the pooled rows this lane's query sees
     const int64_t pr0 = p.pool > 0 ? p.pool_row0[s] : 0;
     const float capl = p.softcap * 1.4426950408889634f;
-    for (int it = -pool_steps;; ++it) {
-        const bool seg = it < 0;  // the pooled rows come first
-        const int j0 = seg ? (it + pool_steps) * MKT : key_lo + it * MKT;
+    for (int v = v_lo; v < v_hi; ++v) {
+        const bool seg = v < pool_steps;  // the pooled rows come first
+        const int j0 = seg ? v * MKT : key_lo + (v - pool_steps) * MKT;
         const int n_here = seg ? n_pool : n_keys;
-        if (!seg) {
-            if (j0 >= n_keys) break;
-            if (j0 + MKT <= win_lo && j0 >= p.keep_first) continue;  // block-uniform: no row sees a key of this step
-        }
+        if (!seg && j0 + MKT <= win_lo && j0 >= p.keep_first) continue;  // block-uniform: no row sees a key of this step
         const bf16_t* Kp = seg ? (const bf16_t*)p.PK : K1;
         const bf16_t* Vp = seg ? (const bf16_t*)p.PV : V;
         const int64_t kr = seg ? pr0 : k1r0, vr = seg ? pr0 : vr0, ldk = seg ? p.ldp : p.ldk1, ldvv = seg ? p.ldp : p.ldv;

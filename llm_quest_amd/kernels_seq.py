@@ -280,7 +280,11 @@ def latent_attn(q, k1, k2, v, out, H, hm, D1, D2, DV, q_hs, k1_hs, v_hs, o_hs, d
     if mfma and D1 + D2 <= 320 and DV <= 256 and max_keys and (not window or window >= max_keys or plain_window):
         head_tiles = -(-H // hm)
         tile_tokens = min(max_new, -(-128 // hm))
-        splits = attn_key_splits(n_seq, head_tiles, max_new, hm, min(max_keys, window + tile_tokens - 1), 128) if plain_window else attn_key_splits(n_seq, head_tiles, max_new, hm, max_keys)
+        if plain_window:  # what a tile walks: its window, and one pooled row per block before it
+            rows = min(max_keys, window + tile_tokens - 1) + (max(0, max_keys - window) // pool if pool else 0)
+            splits = attn_key_splits(n_seq, head_tiles, max_new, hm, rows, 128)
+        else:
+            splits = attn_key_splits(n_seq, head_tiles, max_new, hm, max_keys)
         if splits > 1:
             dvp = 32 if DV <= 32 else 64 if DV <= 64 else 128 if DV <= 128 else 256
             ws = torch.empty(n_seq * head_tiles * -(-max_new * hm // 128) * splits * 128 * (2 + dvp), dtype=F32, device=v.device)

@@ -490,3 +490,12 @@ def test_one_token_steps_deal_a_long_windows_keys_to_several_workgroups(dt, size
     hot = [899 - size, 900 - size, 901 - size, 902 - size, 640, 898, 3, 40]
     (got, want), = _attention_alone(dt, 4, 2, 32, 48, size, pool, torch.tensor([0.5, -1.0, 2.0, 0.0]), 0.0, [[900]] + [[1]] * 4, hot, seed=7)
     assert row_err(got[900:], want[900:]) < ATT_TOL[dt] and row_err(got, want) < ATT_TOL[dt]
+
+
+def test_one_token_steps_deal_many_pooled_rows_too():
+    """4 000 cached keys, blocks of 4 tokens, a window of 100: a one-token step sees some 970 pooled rows and 100 keys; the bf16 kernel deals the pooled rows and
+    the window to several workgroups.  Hot keys far back come through only as a quarter of their block's mean."""
+    hot = [7, 1001, 2500, 3890, 3898, 3899, 3900, 3901]
+    (got, want), = _attention_alone("bfloat16", 2, 1, 32, 48, 100, 4, torch.tensor([0.5, -1.0]), 0.0, [[4000]] + [[1]] * 3, hot, seed=9)
+    assert row_err(got[4000:], want[4000:]) < ATT_TOL["bfloat16"]
+    assert row_err(got[3000:], want[3000:]) < ATT_TOL["bfloat16"]
