@@ -1,0 +1,284 @@
+"""Plain PyTorch-CPU oracle of the Gepilix decoder (test infrastructure only, one function per mechanism).
+
+Gepilix is a pre-norm decoder, x <- x + s1 * mixer(n1(x)), then x <- x + s2 * ff(n2(x)) with per-channel layer scales s1 / s2, whose norms are Dynamic
+Tanh (tanh(alpha x) w + b: no statistics at all).  Mixers:
+  * *parallel*   -- chunked grouped-query softmax attention (biases, no rotation, tanh-capped scores, one sigmoid gate per head) beside a real-gated
+    linear recurrent unit (GELU branch, short convolution, block-diagonal gates); each branch RMS-normed over the width, the mean of the two;
+  * *parallel_2* -- sliding-window grouped-query attention (rotate-half rotary with long-context frequency scaling, capped scores) beside a
+    state-space-duality layer (scalar decay per head, state N x vdim, gate before a grouped norm); a weighted sum of the two;
+  * *wkv*        -- token-shifted linear attention with a data-dependent decay per key channel and a bonus for the current token.
+Feed-forward: down(relu(up x)^2), or top-k routed SiLU-gated experts (weights = softmax over the chosen logits) plus a shared expert.
+
+Everything here works on ONE whole sequence, in the dtype of the tensors handed in (fp32 or fp64), token by token where a recurrence is involved, and
+shares no code with ``llm_quest_amd``.  ``weights`` maps the checkpoint's tensor names to tensors; ``cfg`` is the parsed ``config.json``.
+"""
+
+import math
+
+import torch
+
+
+def dyn_tanh(x, alpha, w, b):
+    return torch.tanh(alpha * x) * w + b
+
+
+def unit_rms(x, eps):
+    return x / torch.sqrt((x * x).mean(dim=-1, keepdim=True) + eps)
+
+
+def gelu_tanh(z):
+    return 0.5 * z * (1.0 + torch.tanh(math.sqrt(2.0 / math.pi) * (z + 0.044715 * z ** 3)))
+
+
+def silu(z):
+    return z * torch.sigmoid(z)
+
+
+def softplus(z):
+    return torch.where(z > 30, z, torch.log1p(torch.exp(torch.clamp(z, max=30.0))))
+
+
+def causal_conv(h, w, b):
+    """h [T, C], w [C, taps], b [C]: y_t = b + sum_j w[:, j] h_(t - taps + 1 + j), zeros before the first token."""
+    T, C = h.shape
+    taps = w.shape[1]
+    y = b.expand(T, C).clone()
+    for t in range(T):
+        for j in range(taps):
+            s = t - taps + 1 + j
+            if s >= 0:
+                y[t] += w[:, j] * h[s]
+    return y
+
+
+def scaled_frequencies(dims, base, scaling):
+    """f_i = base^(-2i/dims); with ``scaling`` {factor, low, high, original}: wavelengths shorter than original/high stay, longer than original/low are
+    divided by factor, between the two the frequencies are blended linearly in original/wavelength."""
+    f = [float(base) ** (-2.0 * i / dims) for i in range(dims // 2)]
+    if not scaling:
+        return f
+    fac, lo, hi, orig = float(scaling["factor"]), float(scaling["low"]), float(scaling["high"]), float(scaling["original"])
+    out = []
+    for x in f:
+        wl = 2.0 * math.pi / x
+        if wl < orig / hi:
+            out.append(x)
+        elif wl > orig / lo:
+            out.append(x / fac)
+        else:
+            s = (orig / wl - lo) / (hi - lo)
+            out.append((1.0 - s) * x / fac + s * x)
+    return out
+
+
+def rotary_half(x, dims, freqs):
+    """x [T, H, D], positions 0 .. T-1: entry i of the first ``dims`` pairs with entry i + dims/2."""
+    T = x.shape[0]
+    half = dims // 2
+    out = x.clone()
+    pos = torch.arange(T, dtype=torch.float64)
+    for i in range(half):
+        ang = (pos * freqs[i]).to(x.dtype) if x.dtype == torch.float64 else (pos.to(torch.float32) * torch.tensor(freqs[i], dtype=torch.float32))
+        c, s = torch.cos(ang)[:, None].to(x.dtype), torch.sin(ang)[:, None].to(x.dtype)
+        u, v = x[:, :, i], x[:, :, i + half]
+        out[:, :, i] = u * c - v * s
+        out[:, :, i + half] = v * c + u * s
+    return out
+
+
+def masked_attention(q, k, v, scale, softcap, visible):
+    """q [T, H, d], k [T, G, d], v [T, G, dv]; ``visible(i, j)`` for j <= i.  Scores times scale, then cap * tanh(score / cap) if cap > 0."""
+    T, H, d = q.shape
+    G = k.shape[1]
+    out = torch.zeros(T, H, v.shape[-1], dtype=q.dtype)
+    for h in range(H):
+        g = h // (H // G)
+        for i in range(T):
+            js = [j for j in range(i + 1) if visible(i, j)]
+            s = (k[js, g] @ q[i, h]) * scale
+            if softcap:
+                s = softcap * torch.tanh(s / softcap)
+            p = torch.softmax(s, dim=0)
+            out[i, h] = p @ v[js, g]
+    return out
+
+
+def chunk_visible(size):
+    return lambda i, j: i // size == j // size
+
+
+def window_visible(size):
+    return lambda i, j: i - j < size
+
+
+def attention_branch(h, w, p, m, eps):
+    """One softmax-attention branch: projections (biases if the checkpoint has them), optional rotary, mask by config, optional per-head gate."""
+    T = h.shape[0]
+    H, G, d, dv = m["heads"], m.get("kv_heads", m["heads"]), m["dim"], m["vdim"]
+
+    def proj(name):
+        y = h @ w[p + name].T
+        return y + w[p + name + ".b"] if p + name + ".b" in w else y
+
+    q, k, v = proj("q").reshape(T, H, d), proj("k").reshape(T, G, d), proj("v").reshape(T, G, dv)
+    rot = m.get("rot")
+    if rot:
+        fr = scaled_frequencies(rot["dims"], rot["base"], rot.get("scaling"))
+        q, k = rotary_half(q, rot["dims"], fr), rotary_half(k, rot["dims"], fr)
+    return q, k, v
+
+
+def rglru_branch(h, w, p, m):
+    """Recurrent block: y = gelu(W_y h + b), u = conv(W_x h + b); per block r, i = sigmoid(block matrix u + b); a = exp(-8 r softplus(lam));
+    S <- a S + sqrt(1 - a^2) (i u); out = W_o (S y)."""
+    T = h.shape[0]
+    y = gelu_tanh(h @ w[p + "y"].T + w[p + "y.b"])
+    u = causal_conv(h @ w[p + "x"].T + w[p + "x.b"], w[p + "conv"], w[p + "conv.b"])
+    nb = w[p + "ra"].shape[0]
+    C = u.shape[1]
+    ub = u.reshape(T, nb, C // nb)
+    r = torch.sigmoid(torch.einsum("boi,tbi->tbo", w[p + "ra"], ub) + w[p + "ra.b"]).reshape(T, C)
+    g = torch.sigmoid(torch.einsum("boi,tbi->tbo", w[p + "ri"], ub) + w[p + "ri.b"]).reshape(T, C)
+    log_a = -8.0 * r * softplus(w[p + "lam"])
+    a = torch.exp(log_a)
+    S = torch.zeros(C, dtype=h.dtype)
+    out = torch.zeros(T, C, dtype=h.dtype)
+    for t in range(T):
+        S = a[t] * S + torch.sqrt(1.0 - a[t] * a[t]) * g[t] * u[t]
+        out[t] = S
+    return (out * y) @ w[p + "o"].T
+
+
+def ssd_branch(h, w, p, m, eps):
+    """State-space-duality layer: W_in h = [z | x | B | C | dt]; x, B, C through conv + silu; dt = softplus(dt + bias); per head
+    S <- exp(-exp(A_log) dt) S + dt B x^T, y = S^T C + D x; (y silu(z)) RMS-normed in groups, times the weight, W_o."""
+    T = h.shape[0]
+    H, P, N, G, ng = m["heads"], m["vdim"], m["state"], m["groups"], m["norm_groups"]
+    inner = H * P
+    proj = h @ w[p + "in"].T
+    z, xbc, dt = proj[:, :inner], proj[:, inner : 2 * inner + 2 * G * N], proj[:, 2 * inner + 2 * G * N :]
+    xbc = silu(causal_conv(xbc, w[p + "conv"], w[p + "conv.b"]))
+    x = xbc[:, :inner].reshape(T, H, P)
+    B = xbc[:, inner : inner + G * N].reshape(T, G, N)
+    C = xbc[:, inner + G * N :].reshape(T, G, N)
+    dt = softplus(dt + w[p + "dt_bias"])
+    A = torch.exp(w[p + "A_log"])
+    y = torch.zeros(T, H, P, dtype=h.dtype)
+    for hd in range(H):
+        g = hd // (H // G)
+        S = torch.zeros(N, P, dtype=h.dtype)
+        for t in range(T):
+            S = torch.exp(-A[hd] * dt[t, hd]) * S + dt[t, hd] * torch.outer(B[t, g], x[t, hd])
+            y[t, hd] = S.T @ C[t, g] + w[p + "D"][hd] * x[t, hd]
+    y = y.reshape(T, inner) * silu(z)
+    y = unit_rms(y.reshape(T, ng, inner // ng), eps).reshape(T, inner) * w[p + "norm"]
+    return y @ w[p + "o"].T
+
+
+def parallel_mixer(h, w, p, m, eps):
+    L, R = m["left"], m["right"]
+    T = h.shape[0]
+    q, k, v = attention_branch(h, w, p + "left.", L, eps)
+    size = (L.get("mask") or {}).get("size", 0)
+    o = masked_attention(q, k, v, L["scale"], L.get("softcap", 0.0), chunk_visible(size) if size else (lambda i, j: True))
+    gate = torch.sigmoid(h @ w[p + "left.g"].T)  # [T, H]
+    left = (o * gate[:, :, None]).reshape(T, -1) @ w[p + "left.o"].T
+    right = rglru_branch(h, w, p + "right.", R)
+    return 0.5 * (unit_rms(left, eps) * w[p + "left.out"] + unit_rms(right, eps) * w[p + "right.out"])
+
+
+def parallel2_mixer(h, w, p, m, eps):
+    L, R = m["left"], m["right"]
+    T = h.shape[0]
+    q, k, v = attention_branch(h, w, p + "left.", L, eps)
+    size = (L.get("mask") or {}).get("size", 0)
+    o = masked_attention(q, k, v, L["scale"], L.get("softcap", 0.0), window_visible(size) if size else (lambda i, j: True))
+    left = o.reshape(T, -1) @ w[p + "left.o"].T
+    right = ssd_branch(h, w, p + "right.", R, eps)
+    return m["left_scale"] * left + m["right_scale"] * right
+
+
+def wkv_mixer(h, w, p, m, eps):
+    """Token-shifted mixes; r, k, v, gate from their own mix; decay exp(-exp(w0 + W2 tanh(W1 mix_w))); o_t = (S + diag(u) k v^T)^T r, then
+    S <- diag(decay) S + k v^T; heads to unit RMS, times the weight, times silu gate, W_o."""
+    T = h.shape[0]
+    H, d = m["heads"], m["dim"]
+    prev = torch.cat([torch.zeros_like(h[:1]), h[:-1]])
+
+    def mix(s):
+        return h + (prev - h) * w[p + "mu." + s]
+
+    r = (mix("r") @ w[p + "r"].T).reshape(T, H, d)
+    k = (mix("k") @ w[p + "k"].T).reshape(T, H, d)
+    v = (mix("v") @ w[p + "v"].T).reshape(T, H, d)
+    gate = silu(mix("g") @ w[p + "g"].T)
+    dec = torch.exp(-torch.exp(torch.tanh(mix("w") @ w[p + "w1"].T) @ w[p + "w2"].T + w[p + "w0"])).reshape(T, H, d)
+    u = w[p + "u"]
+    o = torch.zeros(T, H, d, dtype=h.dtype)
+    for hd in range(H):
+        S = torch.zeros(d, d, dtype=h.dtype)
+        for t in range(T):
+            kv = torch.outer(k[t, hd], v[t, hd])
+            o[t, hd] = (S + u[hd][:, None] * kv).T @ r[t, hd]
+            S = dec[t, hd][:, None] * S + kv
+    o = unit_rms(o, eps).reshape(T, H * d) * w[p + "norm"] * gate
+    return o @ w[p + "o"].T
+
+
+def dense_ff(h, w, p):
+    return torch.relu(h @ w[p + "up"].T) ** 2 @ w[p + "down"].T
+
+
+def gated_expert(h, w, p):
+    return (silu(h @ w[p + "gate"].T) * (h @ w[p + "up"].T)) @ w[p + "down"].T
+
+
+def moe_ff(h, w, p, mlp):
+    E, top = mlp["router"]["experts"], mlp["router"]["top"]
+    logits = h @ w[p + "router"].T
+    if p + "router.b" in w:
+        logits = logits + w[p + "router.b"]
+    val, idx = torch.topk(logits, top, dim=-1)
+    wt = torch.softmax(val, dim=-1)
+    out = torch.zeros(h.shape[0], w[p + "e0.down"].shape[0], dtype=h.dtype)
+    for t in range(h.shape[0]):
+        for j in range(top):
+            e = int(idx[t, j])
+            out[t] += wt[t, j] * gated_expert(h[t : t + 1], w, f"{p}e{e}.")[0]
+    if mlp.get("shared"):
+        out = out + gated_expert(h, w, p + "shared.")
+    return out
+
+
+def router_choice(h, w, p, mlp):
+    """(chosen expert ids [T, top], gap between the last chosen and the first rejected logit [T]) -- tests skip tokens whose choice is a close call."""
+    logits = h @ w[p + "router"].T
+    if p + "router.b" in w:
+        logits = logits + w[p + "router.b"]
+    s, idx = torch.sort(logits, dim=-1, descending=True)
+    top = mlp["router"]["top"]
+    gap = s[:, top - 1] - s[:, top] if s.shape[1] > top else torch.full((h.shape[0],), float("inf"))
+    return idx[:, :top], gap
+
+
+def forward(cfg, weights, tokens, dtype=torch.float32, return_layers=False):
+    """Logits [T, vocab] of one whole sequence (and the residual stream after every layer)."""
+    w = {k: (v.to(dtype) if v.is_floating_point() else v) for k, v in weights.items()}
+    eps = cfg["norm"]["eps"]
+    x = w["embed"][torch.as_tensor(tokens, dtype=torch.long)]
+    layers = []
+    for i, layer in enumerate(cfg["layers"]):
+        p = f"l{i}."
+        h = dyn_tanh(x, w[p + "norm1.alpha"], w[p + "norm1"], w[p + "norm1.b"])
+        kind = layer["type"]
+        mixer = {"parallel": parallel_mixer, "parallel_2": parallel2_mixer, "wkv": wkv_mixer}[kind]
+        x = x + w[p + "ls1"] * mixer(h, w, p + "mix.", layer["mixer"], eps)
+        mlp = layer.get("mlp")
+        if mlp is not None:
+            h = dyn_tanh(x, w[p + "norm2.alpha"], w[p + "norm2"], w[p + "norm2.b"])
+            y = dense_ff(h, w, p + "mlp.") if mlp["kind"] == "dense" else moe_ff(h, w, p + "mlp.", mlp)
+            x = x + w[p + "ls2"] * y
+        layers.append(x)
+    h = dyn_tanh(x, w["final.norm.alpha"], w["final.norm"], w["final.norm.b"])
+    logits = h @ w["head"].T
+    return (logits, layers) if return_layers else logits
