@@ -544,7 +544,8 @@ int mi355_router_logits(int64_t tokens, int E, int K, const float* x, int64_t ld
 /* Grouped sigmoid router: s = sigmoid(logits), choice = s + correction (may be NULL); a group (E / groups neighbours) scores the sum of its two
  * largest choices, experts outside the `keep` best groups are excluded, the `top` largest choices win; wts = s / (sum + 1e-20) * scale.
  * ids int32 [tokens, top] in descending order of choice, wts fp32 [tokens, top].  mode 1 (softmax router): s = softmax(logits) over all experts, the `top`
- * largest win, wts = their s * scale without renormalisation (correction / groups unused). */
+ * largest win, wts = their s * scale without renormalisation (correction / groups unused).  mode 2: as mode 1 on logits + correction (a bias), the winners'
+ * s divided by their sum, i.e. the softmax over the chosen logits alone, times scale. */
 int mi355_moe_route(int64_t tokens, int E, int top, int groups, int keep, const float* logits, const float* correction, float scale, int mode, int* ids,
                     float* wts, void* stream);
 /* Dispatch lists of `entries` = tokens * top choices: offs int32 [E + 1], perm int32 [entries] = the entries sorted by expert (token order inside one). */
@@ -554,7 +555,7 @@ int mi355_moe_dispatch(int64_t entries, int E, const int* ids, int* offs, int* p
  * a_rows: sorted row r reads A row a_rows[r] / a_div; c_rows: it writes C row c_rows[r]; row_scale: that C row is scaled.  epi 1 = relu(x)^2.
  * use_mfma needs bf16 A and B; otherwise fp32 FMA accumulation in a fixed k order.  bias (fp32 [N], may be NULL) is added to every row before epi.
  * epi 2 / 3 (gated feed-forward): B's rows come in blocks of 64 = [32 gate rows | 32 up rows] (N a multiple of 64), C has n_out <= N / 2 columns,
- * C[m, 32 b + i] = act(gate, up) of block b: 2 = g sigmoid(1.702 g) (u + 1) with g = min(gate, limit), u = clamp(up, -limit, limit); 3 = gelu_tanh(gate) * up. */
+ * C[m, 32 b + i] = act(gate, up) of block b: 2 = g sigmoid(1.702 g) (u + 1) with g = min(gate, limit), u = clamp(up, -limit, limit); 3 = gelu_tanh(gate) * up; 4 = silu(gate) * up. */
 int mi355_bgemm(int batch, int M, int N, int K, const void* A, int a_dt, int64_t lda, int64_t a_bs, const void* B, int b_dt, int64_t sbn, int64_t sbk,
                 int64_t b_bs, void* C, int c_dt, int64_t ldc, int64_t c_bs, const int* grp_offs, const int* a_rows, int a_div, const int* c_rows,
                 const float* row_scale, int epi, int use_mfma, const float* bias, float limit, int n_out, void* stream);
@@ -569,12 +570,13 @@ int mi355_bgemm(int batch, int M, int N, int K, const void* A, int a_dt, int64_t
  * softcap > 0: score <- softcap * tanh(score / softcap) after the scale.  sink (fp32 [H], may be NULL): exp(sink[h]) joins head h's softmax denominator.
  * pool > 0 (needs window > 0, keep_first == 0, D2 == 0): besides the window the query at position i sees one pooled key / value row for every block b of
  * `pool` tokens with (b + 1) * pool <= i - window + 1; block b of sequence s is row pool_row0[s] + b of PK / PV (pitch ldp, head strides k1_hs / v_hs,
- * dtype dt); pooled rows and tokens share one softmax. */
+ * dtype dt); pooled rows and tokens share one softmax.  chunk > 0: positions are cut into chunks of that many, counted from the sequence's first token,
+ * and a query sees only the keys j <= i of its own chunk, floor(j / chunk) == floor(i / chunk) (no kept first tokens, no pooled blocks). */
 int mi355_latent_attn(int n_seq, int max_new, int H, int hm, int D1, int D2, int DV, const float* Q, int64_t ldq, int q_hs, const void* K1, int64_t ldk1,
                       int k1_hs, const void* K2, int64_t ldk2, const void* V, int64_t ldv, int v_hs, void* O, int64_t ldo, int o_hs, int dt,
                       const int* q_row0, const int* n_new, const int* past, const int* k1_row0, const int* k2_row0, const int* v_row0, float scale,
                       int use_mfma, int splits, float* ws, int64_t ws_floats, int kv_rep, int window, int keep_first, float softcap, const float* sink,
-                      int pool, const void* PK, const void* PV, int64_t ldp, const int* pool_row0, void* stream);
+                      int pool, const void* PK, const void* PV, int64_t ldp, const int* pool_row0, int chunk, void* stream);
 
 /* ---- parallel-sublayer hybrid decoders in ragged batches (csrc/seqrec.hip) ---- */
 /* v = x + y1[t] + sum_{p < parts} y2[t * parts + p] (fp32 rows; y1 / y2 of dtype y*_dt, may be NULL); x_out (may be NULL or x) <- v.  For each weight
@@ -586,9 +588,9 @@ int mi355_group_rmsnorm_sum(int64_t tokens, int width, const float* x, const voi
 /* Causal convolution over time on every channel of ragged rows: y[t, c] = (residual ? x[t, c] : 0) + act(sum_j w[c, j] * in(t - taps + 1 + j, c)), w fp32
  * [C, taps] (the last column weighs the current token); inputs before the step's first row come from state[slot[s]] (fp32 [slots, taps - 1, C], the inputs
  * of the sequence's last taps - 1 tokens, zeros before its start), which afterwards holds the step's last inputs.  row_seq[t] = index of t's sequence
- * in the step; act 0 none, 1 silu; taps <= 16. */
+ * in the step; act 0 none, 1 silu; taps <= 16.  bias (fp32 [C], may be NULL) is added to the convolution before the activation. */
 int mi355_ragged_conv(int64_t tokens, int n_seq, int C, int taps, const void* x, int x_dt, int64_t ldx, const float* w, const int* row_seq, const int* seq_off,
-                      const int* slot, float* state, int act, int residual, void* y, int y_dt, int64_t ldy, void* stream);
+                      const int* slot, float* state, int act, int residual, void* y, int y_dt, int64_t ldy, const float* bias, void* stream);
 /* Query / key / value rows of grouped-query attention: src[t] = [H x d | G x d | G x dv] (+ bias fp32, may be NULL); query and key heads get an RMS norm over d
  * (weights qw / kw fp32 [d], NULL: none) and a rotation of their first `dims` entries (layout as mi355_rope_heads); query head h times qscale[h] (may be NULL)
  * goes to q_out fp32 [t, h * d]; key and value heads go to cache row dst_row[t] = [G x d | G x dv] of dtype c_dt.  qt_every > 0: the query at position p
@@ -606,7 +608,7 @@ int mi355_delta_rule_ragged(int64_t tokens, int n_seq, const int* seq_off, const
                             int64_t ldq, int64_t ldk, const void* v, int v_dt, int64_t ldv, const void* b, const void* a, int ba_dt, int64_t ldb, int64_t lda,
                             const float* A_log, const float* dt_bias, float qscale, float* state, float* o, float* ws, void* stream);
 /* Gated feed-forward activation on rows [gate (F) | up (F)] -> [F].  kind 0: gelu_tanh(gate) * up.  kind 1: g = min(gate, limit), u = clamp(up, -limit, limit),
- * g * sigmoid(1.702 g) * (u + 1). */
+ * g * sigmoid(1.702 g) * (u + 1).  kind 2: silu(gate) * up. */
 int mi355_glu_rows(int64_t rows, int F, const void* in, int in_dt, int64_t ld_in, int kind, float limit, void* out, int out_dt, int64_t ld_out, void* stream);
 
 /* ---- decoders with sandwich norms in ragged batches (csrc/seqsand.hip) ---- */
@@ -622,6 +624,36 @@ int mi355_pool_rows_update(int n_seq, int max_blocks, int width, int pool, const
  * kind 1: out = x * sigmoid(gate), gate rows of dtype g_dt and pitch ldg (params unused). */
 int mi355_act_rows(int64_t rows, int n, const void* x, int x_dt, int64_t ldx, const void* gate, int g_dt, int64_t ldg, int kind, const float* params, void* out,
                    int out_dt, int64_t ldo, void* stream);
+
+/* ---- decoders with side-by-side branches and statistic-free norms in ragged batches (csrc/seqpar.hip) ---- */
+/* y = ca * N_a(ya[t]) + cb * N_b(yb[t]) + sum_{p < parts} y2[t * parts + p], N(y) = y / sqrt(mean(y^2) + eps) * w_n where the branch has a weight (wa / wb, fp32
+ * [width], may be NULL: N(y) = y); any of ya / yb / y2 may be NULL.  v = x[t] + ls * y (ls fp32 [width], NULL: 1); x_out (may be NULL or x) <- v;
+ * out (dtype out_dt) and out32 (fp32), each may be NULL <- tanh(alpha * v) * w + b (w, b fp32 [width], both NULL: no norm). */
+int mi355_dyt_sum(int64_t tokens, int width, const float* x, const void* ya, int ya_dt, int64_t ldya, const float* wa, float ca, const void* yb, int yb_dt,
+                  int64_t ldyb, const float* wb, float cb, const void* y2, int y2_dt, int64_t ldy2, int parts, const float* ls, float eps, float* x_out, float alpha,
+                  const float* w, const float* b, void* out, int out_dt, float* out32, void* stream);
+/* Token shift: out[t, s * C + c] = h[t, c] + (h'[t, c] - h[t, c]) * mu[s * C + c], s < n_mix, h' the previous token's row of the sequence (this step's, or
+ * state[slot] fp32 [slots, C] for the step's first row; zeros at a sequence's start); afterwards state[slot] <- the step's last row. */
+int mi355_token_shift(int64_t tokens, int n_seq, int C, int n_mix, const float* h, int64_t ldh, const float* mu, const int* row_seq, const int* seq_off,
+                      const int* slot, float* state, void* out, int out_dt, int64_t ldo, void* stream);
+/* Linear recurrence over a matrix state per head, state fp32 [slots, H, dk, dv], o fp32 [tokens, H * dv]; query / key head of value head h: h / qk_rep.
+ * post 0: o_t = S^T q_t + (sum_i q_i u_i k_i) v_t, then S <- diag(exp(-exp(z[t, h, :]))) S + k_t v_t^T (z fp32 rows [H * dk], u fp32 [H * dk]).
+ * post 1: dt = softplus(z[t, h] + dt_bias[h]) (z fp32 rows [H]); S <- exp(-exp(A_log[h]) dt) S + k_t (dt v_t)^T; o_t = S^T q_t + D[h] v_t.  dk <= 256. */
+int mi355_linrec_ragged(int n_seq, const int* seq_off, const int* slot, int H, int qk_rep, int dk, int dv, const void* q, const void* k, int q_dt, int64_t ldq,
+                        int64_t ldk, const void* v, int v_dt, int64_t ldv, const float* z, int64_t ldz, int post, const float* u, const float* dt_bias,
+                        const float* A_log, const float* D, float* state, float* o, void* stream);
+/* Real-gated linear recurrent unit, per channel c of block b = c / n (n = C / blocks), j = c % n: r = sigmoid(gates[t, 2 n b + j] + gbias[2 n b + j]),
+ * i = sigmoid(gates[t, 2 n b + n + j] + gbias[2 n b + n + j]) (gbias fp32 [2 C], may be NULL); a = exp(-decay_c r softplus(lam[c])); S <- a S + sqrt(1 - a^2) i u[t, c]; out[t, c] = S gelu_tanh(y[t, c]).
+ * u, gates fp32 rows; state fp32 [slots, C]. */
+int mi355_rglru_ragged(int n_seq, int C, int blocks, float decay_c, const float* u, int64_t ldu, const float* gates, int64_t ldg, const float* gbias, const float* lam,
+                       const void* y, int y_dt, int64_t ldy, const int* seq_off, const int* slot, float* state, void* out, int out_dt, int64_t ldo, void* stream);
+/* RMS norm in `groups` equal consecutive groups of fp32 rows o [n] with weight w fp32 [n] and a SiLU gate: gate_first 0: o / rms(o) * w * silu(gate);
+ * gate_first 1: g = o silu(gate), g / rms(g) * w. */
+int mi355_gated_groupnorm(int64_t tokens, int n, int groups, const float* o, int64_t ldo_in, const float* w, const void* gate, int g_dt, int64_t ldg, int gate_first,
+                          float eps, void* out, int out_dt, int64_t ldo, void* stream);
+/* Rows [n] -> [n].  kind 0: relu(x)^2; 1: tanh(x); 2: x[r, i] * sigmoid(gate[r, i / group]) (one gate per run of `group` entries). */
+int mi355_unary_rows(int64_t rows, int n, const void* x, int x_dt, int64_t ldx, int kind, const void* gate, int g_dt, int64_t ldg, int group, void* out,
+                     int out_dt, int64_t ldo, void* stream);
 
 #ifdef __cplusplus
 }

@@ -113,10 +113,10 @@ SIGNATURES = {
     "mi355_moe_route": [_L, _I, _I, _I, _I, _P, _P, _F, _I, _P, _P, _P],
     "mi355_moe_dispatch": [_L, _I, _P, _P, _P, _P],
     "mi355_bgemm": [_I, _I, _I, _I, _P, _I, _L, _L, _P, _I, _L, _L, _L, _P, _I, _L, _L, _P, _P, _I, _P, _P, _I, _I, _P, _F, _I, _P],
-    "mi355_latent_attn": [_I, _I, _I, _I, _I, _I, _I, _P, _L, _I, _P, _L, _I, _P, _L, _P, _L, _I, _P, _L, _I, _I, _P, _P, _P, _P, _P, _P, _F, _I, _I, _P, _L, _I, _I, _I, _F, _P, _I, _P, _P, _L, _P, _P],
+    "mi355_latent_attn": [_I, _I, _I, _I, _I, _I, _I, _P, _L, _I, _P, _L, _I, _P, _L, _P, _L, _I, _P, _L, _I, _I, _P, _P, _P, _P, _P, _P, _F, _I, _I, _P, _L, _I, _I, _I, _F, _P, _I, _P, _P, _L, _P, _I, _P],
     # parallel-sublayer hybrid decoders in ragged batches (csrc/seqrec.hip)
     "mi355_group_rmsnorm_sum": [_L, _I, _P, _P, _I, _L, _P, _I, _L, _I, _P, _I, _F, _P, _P, _I, _P, _P, _P, _I, _P, _P],
-    "mi355_ragged_conv": [_L, _I, _I, _I, _P, _I, _L, _P, _P, _P, _P, _P, _I, _I, _P, _I, _L, _P],
+    "mi355_ragged_conv": [_L, _I, _I, _I, _P, _I, _L, _P, _P, _P, _P, _P, _I, _I, _P, _I, _L, _P, _P],
     "mi355_qkv_rows_append": [_L, _I, _I, _I, _I, _P, _I, _L, _P, _P, _P, _F, _P, _I, _I, _P, _P, _P, _P, _L, _P, _I, _L, _F, _I, _P, _L, _F, _P],
     "mi355_delta_rule_ragged": [_L, _I, _P, _P, _I, _I, _I, _I, _P, _P, _I, _L, _L, _P, _I, _L, _P, _P, _I, _L, _L, _P, _P, _F, _P, _P, _P, _P],
     "mi355_glu_rows": [_L, _I, _P, _I, _L, _I, _F, _P, _I, _L, _P],
@@ -124,6 +124,13 @@ SIGNATURES = {
     "mi355_sandwich_rmsnorm": [_L, _I, _P, _P, _I, _L, _P, _P, _P, _F, _P, _I, _P],
     "mi355_pool_rows_update": [_I, _I, _I, _I, _P, _I, _L, _P, _I, _L, _P, _P, _P, _P, _P],
     "mi355_act_rows": [_L, _I, _P, _I, _L, _P, _I, _L, _I, _P, _P, _I, _L, _P],
+    # decoders with side-by-side branches and statistic-free norms in ragged batches (csrc/seqpar.hip)
+    "mi355_dyt_sum": [_L, _I, _P, _P, _I, _L, _P, _F, _P, _I, _L, _P, _F, _P, _I, _L, _I, _P, _F, _P, _F, _P, _P, _P, _I, _P, _P],
+    "mi355_token_shift": [_L, _I, _I, _I, _P, _L, _P, _P, _P, _P, _P, _P, _I, _L, _P],
+    "mi355_linrec_ragged": [_I, _P, _P, _I, _I, _I, _I, _P, _P, _I, _L, _L, _P, _I, _L, _P, _L, _I, _P, _P, _P, _P, _P, _P, _P],
+    "mi355_rglru_ragged": [_I, _I, _I, _F, _P, _L, _P, _L, _P, _P, _P, _I, _L, _P, _P, _P, _P, _I, _L, _P],
+    "mi355_gated_groupnorm": [_L, _I, _I, _P, _L, _P, _P, _I, _L, _I, _F, _P, _I, _L, _P],
+    "mi355_unary_rows": [_L, _I, _P, _I, _L, _I, _P, _I, _L, _I, _P, _I, _L, _P],
     # measurement aid (csrc/probe.hip)
     "mi355_mfma_pipe_probe": [_I, _I, _P, _P],
     # stand-alone RoPE and dropout (csrc/rope_dropout.hip, csrc/attention_generic.hip)

@@ -31,20 +31,21 @@ struct BgemmArgs {
     const int* c_rows;       // or null: sorted row r writes C row c_rows[r]
     const float* row_scale;  // or null: C row (after c_rows) is multiplied by row_scale[that row]
     const float* bias;       // or null: bias[n] is added to column n before the epilogue
-    int epi;                 // 0 none, 1 relu(x)^2, 2 / 3 gated (see gated_act): B's rows come in blocks of 64 = [32 gate rows | 32 up rows], C has n_out columns
+    int epi;                 // 0 none, 1 relu(x)^2, 2 / 3 / 4 gated (see gated_act): B's rows come in blocks of 64 = [32 gate rows | 32 up rows], C has n_out columns
     float limit;
     int n_out;
     int a_dt, b_dt, c_dt;
 };
 
 // Gated activations of a feed-forward's [gate | up] product.  2: g = min(gate, limit), u = clamp(up, -limit, limit), g sigmoid(1.702 g) (u + 1).
-// 3: gelu_tanh(gate) * up.
+// 3: gelu_tanh(gate) * up.  4: silu(gate) * up.
 __device__ __forceinline__ float gated_act(int epi, float g, float u, float limit) {
     if (epi == 2) {
         g = fminf(g, limit);
         u = fminf(fmaxf(u, -limit), limit);
         return g / (1.0f + expf(-1.702f * g)) * (u + 1.0f);
     }
+    if (epi == 4) return g / (1.0f + expf(-g)) * u;
     return 0.5f * g * (1.0f + tanhf(0.7978845608028654f * (g + 0.044715f * g * g * g))) * u;
 }
 
@@ -359,7 +360,7 @@ extern "C" int mi355_bgemm(int batch, int M, int N, int K, const void* A, int a_
     MI355_REQUIRE(batch > 0 && batch <= 65535 && M > 0 && N > 0 && K > 0 && A && B && C, "bgemm: bad arguments");
     MI355_REQUIRE((a_dt == MI355_DT_BF16 || a_dt == MI355_DT_F32) && (b_dt == MI355_DT_BF16 || b_dt == MI355_DT_F32) && (c_dt == MI355_DT_BF16 || c_dt == MI355_DT_F32),
                   "bgemm: bad dtype");
-    MI355_REQUIRE(epi >= 0 && epi <= 3, "bgemm: bad epilogue");
+    MI355_REQUIRE(epi >= 0 && epi <= 4, "bgemm: bad epilogue");
     MI355_REQUIRE(epi < 2 || (N % 64 == 0 && n_out > 0 && n_out <= N / 2 && !bias), "bgemm: a gated epilogue takes B rows in [32 gate | 32 up] blocks (N a multiple of 64), n_out <= N / 2 columns, no bias");
     MI355_REQUIRE(!a_rows || a_div >= 1, "bgemm: gathered rows need a divisor >= 1");
     MI355_REQUIRE(sbn >= 1 && sbk >= 1 && (sbn == 1 || sbk == 1), "bgemm: one of B's strides must be 1");

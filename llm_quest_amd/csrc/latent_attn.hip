@@ -34,6 +34,7 @@ struct LatAttnArgs {
     int kv_rep;  // query heads per key / value head (grouped queries): head h reads key / value head h / kv_rep
     int window;  // > 0: a query at position i sees key j <= i only if i - j < window or j < keep_first (sliding window that keeps the first tokens)
     int keep_first;
+    int chunk;  // > 0: positions are cut into chunks of this many, counted from the sequence's first token; a query sees only the keys of its own chunk
     float softcap;      // > 0: score <- softcap * tanh(score / softcap) after the scale
     const float* sink;  // fp32 [H] or NULL: exp(sink[h]) joins the denominator of head h (no key, no value, not scaled)
     int pool;           // > 0: one pooled key / value row per `pool` tokens (needs window > 0, D2 == 0); rows PK / PV, first row of sequence s = pool_row0[s]
@@ -51,7 +52,14 @@ __device__ __forceinline__ int pooled_visible(int lim, int window, int pool) {
 __device__ __forceinline__ float cap_score(float s, float cap) { return cap > 0.f ? cap * tanhf(s / cap) : s; }
 
 // key j for the query at position lim (lim < 0: a padding row that sees nothing)
-__device__ __forceinline__ bool key_visible(int j, int lim, int window, int keep_first) { return j <= lim && (window <= 0 || lim - j < window || j < keep_first); }
+__device__ __forceinline__ bool key_visible(int j, int lim, int window, int keep_first, int chunk) {
+    return j <= lim && (window <= 0 || lim - j < window || j < keep_first) && (chunk <= 0 || j >= lim / chunk * chunk);
+}
+// keys below this one are seen by no row of a tile whose first row stands at position pos0 (rows of a tile are consecutive positions)
+__device__ __forceinline__ int tile_key_floor(int pos0, int window, int chunk) {
+    const int w = window > 0 ? pos0 - window + 1 : 0, c = chunk > 0 ? pos0 / chunk * chunk : 0;
+    return max(w, c);
+}
 
 __device__ __forceinline__ float lda_dt(const void* p, int dt, int64_t i) { return dt == MI355_DT_F32 ? ((const float*)p)[i] : bf2f(((const bf16_t*)p)[i]); }
 
@@ -90,7 +98,7 @@ __global__ __launch_bounds__(256) void latent_attn_fma_kernel(LatAttnArgs p) {
         for (int i = 0; i < NC; ++i) o[r][i] = 0.f;
 
     const int kvh = head0 / p.kv_rep;
-    const int win_lo = p.window > 0 ? past + tok0 - p.window + 1 : 0;  // keys below it are outside the window of every row of the tile
+    const int win_lo = tile_key_floor(past + tok0, p.window, p.chunk);  // keys below it are outside the window (or chunk) of every row of the tile
     const int n_pool = p.pool > 0 ? pooled_visible(n_keys - 1, p.window, p.pool) : 0;  // pooled rows any row of the tile may see
     const int pool_steps = (n_pool + AN - 1) / AN;
     const int64_t pr0 = p.pool > 0 ? p.pool_row0[s] : 0;
@@ -144,7 +152,7 @@ __global__ __launch_bounds__(256) void latent_attn_fma_kernel(LatAttnArgs p) {
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 const int j = j0 + tx + 16 * i;
-                const bool vis = seg ? j < npv[a] : key_visible(j, lim[a], p.window, p.keep_first);
+                const bool vis = seg ? j < npv[a] : key_visible(j, lim[a], p.window, p.keep_first, p.chunk);
                 acc[a][i] = vis ? cap_score(acc[a][i] * p.scale, p.softcap) : -__builtin_huge_valf();
                 mx = fmaxf(mx, acc[a][i]);
             }
@@ -267,12 +275,12 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(LatAttnArgs p, in
         }
     }
     const int n_keys = past + min(tok0 + tm, n_new);
-    const int win_lo = p.window > 0 ? past + tok0 - p.window + 1 : 0;  // keys below it are outside the window of every row of the tile
+    const int win_lo = tile_key_floor(past + tok0, p.window, p.chunk);  // keys below it are outside the window (or chunk) of every row of the tile
     // The tile's work is a list of 64-row steps: first the pooled rows any of its rows may see, then the keys from key_lo on (under a plain window dealt
     // out to several workgroups that is the window's lower edge, else 0: steps below a window are skipped one by one).  Workgroup `split` takes its share.
     const int n_pool = p.pool > 0 ? pooled_visible(n_keys - 1, p.window, p.pool) : 0;
     const int pool_steps = (n_pool + MKT - 1) / MKT;
-    const int key_lo = (p.splits > 1 && p.window > 0 && p.keep_first == 0 && win_lo > 0) ? win_lo / MKT * MKT : 0;
+    const int key_lo = (p.splits > 1 && p.keep_first == 0 && win_lo > 0) ? win_lo / MKT * MKT : 0;
     const int all_steps = pool_steps + (n_keys - key_lo + MKT - 1) / MKT;
     int v_lo = 0, v_hi = all_steps;
     if (p.splits > 1) {
@@ -366,7 +374,7 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(LatAttnArgs p, in
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
                 const int j = j0 + kb * 32 + 8 * (r >> 2) + 4 * hf + (r & 3);
-                const bool vis = seg ? j < npv : (key_visible(j, lim, p.window, p.keep_first) && j < n_keys);
+                const bool vis = seg ? j < npv : (key_visible(j, lim, p.window, p.keep_first, p.chunk) && j < n_keys);
                 const float v = !vis ? NEG : (p.softcap > 0.f ? capl * tanhf(sacc[kb][r] * p.scale / p.softcap) : sacc[kb][r] * sc2);
                 sacc[kb][r] = v;
                 mx = fmaxf(mx, v);
@@ -481,7 +489,7 @@ extern "C" int mi355_latent_attn(int n_seq, int max_new, int H, int hm, int D1, 
                                  int k1_hs, const void* K2, int64_t ldk2, const void* V, int64_t ldv, int v_hs, void* O, int64_t ldo, int o_hs, int dt,
                                  const int* q_row0, const int* n_new, const int* past, const int* k1_row0, const int* k2_row0, const int* v_row0, float scale,
                                  int use_mfma, int splits, float* ws, int64_t ws_floats, int kv_rep, int window, int keep_first, float softcap, const float* sink,
-                                 int pool, const void* PK, const void* PV, int64_t ldp, const int* pool_row0, void* stream) {
+                                 int pool, const void* PK, const void* PV, int64_t ldp, const int* pool_row0, int chunk, void* stream) {
     MI355_REQUIRE(n_seq > 0 && n_seq <= 65535 && max_new > 0 && H > 0 && D1 > 0 && D2 >= 0 && DV > 0 && DV <= 512 && Q && K1 && V && O && (D2 == 0 || K2),
                   "latent_attn: bad arguments (value width <= 512)");
     MI355_REQUIRE(dt == MI355_DT_BF16 || dt == MI355_DT_F32, "latent_attn: bad dtype");
@@ -490,6 +498,7 @@ extern "C" int mi355_latent_attn(int n_seq, int max_new, int H, int hm, int D1, 
                   "latent_attn: several heads per tile (a power of two <= 32) need shared keys and values (head stride 0, or one key / value head for the tile's heads)");
     MI355_REQUIRE(!use_mfma || dt == MI355_DT_BF16, "latent_attn: the MFMA path takes bf16 keys and values");
     MI355_REQUIRE(softcap >= 0.f && pool >= 0, "latent_attn: bad softcap or pool");
+    MI355_REQUIRE(chunk >= 0 && (chunk == 0 || (keep_first == 0 && pool == 0)), "latent_attn: chunks combine with neither kept first tokens nor pooled blocks");
     MI355_REQUIRE(pool == 0 || (window > 0 && keep_first == 0 && D2 == 0 && PK && PV && pool_row0 && ldp >= (int64_t)((H - 1) / kv_rep) * k1_hs + D1 &&
                                 ldp >= (int64_t)((H - 1) / kv_rep) * v_hs + DV),
                   "latent_attn: pooled blocks need a window, one-part keys and the pooled rows (laid out like the key / value rows)");
@@ -504,7 +513,7 @@ extern "C" int mi355_latent_attn(int n_seq, int max_new, int H, int hm, int D1, 
     p.D1 = D1, p.D2 = D2, p.DV = DV, p.H = H, p.hm = hm, p.dt = dt;
     p.q_row0 = q_row0, p.n_new = n_new, p.past = past, p.k1_row0 = k1_row0, p.k2_row0 = k2_row0, p.v_row0 = v_row0;
     p.scale = scale;
-    p.kv_rep = kv_rep, p.window = window, p.keep_first = keep_first;
+    p.kv_rep = kv_rep, p.window = window, p.keep_first = keep_first, p.chunk = chunk;
     p.softcap = softcap, p.sink = sink, p.pool = pool, p.PK = PK, p.PV = PV, p.ldp = ldp, p.pool_row0 = pool_row0;
     p.splits = 1, p.ws = nullptr;
     const bool mfma = use_mfma && D1 + D2 <= 320 && DV <= 256;  // what the MFMA kernel keeps in registers; larger heads take the FMA path

@@ -545,6 +545,8 @@ extern "C" int mi355_router_logits(int64_t tokens, int E, int K, const float* x,
 // choice scores; only experts of the `keep` best groups may be chosen; the `top` largest allowed choice scores win (ties: lowest index).
 // weights = s of the winners / (their sum + 1e-20) * scale.  One wave per token, expert e on lane e % 64, register e / 64.
 // mode 1 (softmax router): s = softmax(logits) over ALL experts, choice = s (no correction, no groups), weights = s of the winners * scale, not renormalised.
+// mode 2 (softmax over the winners): as mode 1 on logits + correction (a bias that counts for choice and weight), the winners' s divided by their sum --
+// the softmax over the chosen logits alone -- times scale.
 template <int EPL>
 __global__ __launch_bounds__(256) void moe_route_kernel(int64_t T, int E, int top, int groups, int keep, const float* __restrict__ logits, const float* __restrict__ corr,
                                                         float scale, int mode, int* __restrict__ ids, float* __restrict__ wts) {
@@ -552,12 +554,12 @@ __global__ __launch_bounds__(256) void moe_route_kernel(int64_t T, int E, int to
     const float NEG = -__builtin_huge_valf();
     for (int64_t t = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6); t < T; t += (int64_t)gridDim.x * 4) {
         float s[EPL], c[EPL];
-        if (mode == 1) {
+        if (mode >= 1) {
             float mx = NEG;
 #pragma unroll
             for (int j = 0; j < EPL; ++j) {
                 const int e = lane + 64 * j;
-                s[j] = e < E ? logits[t * E + e] : NEG;
+                s[j] = e < E ? logits[t * E + e] + (mode == 2 && corr ? corr[e] : 0.f) : NEG;
                 mx = fmaxf(mx, s[j]);
             }
             mx = wave_max(mx);
@@ -587,7 +589,7 @@ __global__ __launch_bounds__(256) void moe_route_kernel(int64_t T, int E, int to
                 }
             }
         }
-        if (mode != 1 && groups > 1) {
+        if (mode == 0 && groups > 1) {
             const int per = E / groups;
             // group scores: lane g keeps the score of group g (+ 64 * register)
             float gs[EPL];
@@ -685,7 +687,7 @@ __global__ __launch_bounds__(256) void moe_route_kernel(int64_t T, int E, int to
 
 extern "C" int mi355_moe_route(int64_t tokens, int E, int top, int groups, int keep, const float* logits, const float* correction, float scale, int mode, int* ids,
                                float* wts, void* stream) {
-    MI355_REQUIRE(tokens > 0 && E > 0 && E <= 512 && top > 0 && top <= E && logits && ids && wts && (mode == 0 || mode == 1), "moe_route: bad arguments (experts <= 512)");
+    MI355_REQUIRE(tokens > 0 && E > 0 && E <= 512 && top > 0 && top <= E && logits && ids && wts && mode >= 0 && mode <= 2, "moe_route: bad arguments (experts <= 512)");
     MI355_REQUIRE(groups >= 1 && E % groups == 0 && keep >= 1 && keep <= groups && (int64_t)keep * (E / groups) >= top, "moe_route: the kept groups must hold the experts to choose");
     const int grid = rows_grid(tokens, 4);
     if (E <= 64) moe_route_kernel<1><<<grid, 256, 0, ST(stream)>>>(tokens, E, top, groups, keep, logits, correction, scale, mode, ids, wts);

@@ -206,11 +206,13 @@ extern "C" int mi355_group_rmsnorm_sum(int64_t tokens, int width, const float* x
 // ------------------------------------------------------------------------------------------- short causal convolution over time, ragged, carried state
 // y[t, c] = (residual ? x[t, c] : 0) + act( sum_{j < taps} w[c, j] * in(t - taps + 1 + j, c) ): in(.) is the same sequence's row of this step, or -- before
 // the step's first row -- the carried state: state[slot, i, c] (fp32 [slots, taps - 1, C]) holds the input taps - 1 - i tokens before the step's first
-// one (zeros before the sequence's start).  act: 0 none, 1 silu.  Afterwards the state takes the step's last taps - 1 inputs.
+// one (zeros before the sequence's start).  act: 0 none, 1 silu.  bias (fp32 [C], may be null) is added to the convolution before the activation.
+// Afterwards the state takes the step's last taps - 1 inputs.
 #define CONV_MAX_TAPS 16
 __global__ __launch_bounds__(256) void ragged_conv_kernel(int64_t T, int C, int taps, const void* __restrict__ x, int x_dt, int64_t ldx, const float* __restrict__ w,
                                                           const int* __restrict__ row_seq, const int* __restrict__ seq_off, const int* __restrict__ slot,
-                                                          const float* __restrict__ state, int act, int residual, void* __restrict__ y, int y_dt, int64_t ldy) {
+                                                          const float* __restrict__ state, int act, int residual, void* __restrict__ y, int y_dt, int64_t ldy,
+                                                          const float* __restrict__ bias) {
     const int64_t total = T * C;
     for (int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; e < total; e += (int64_t)gridDim.x * blockDim.x) {
         const int64_t t = e / C;
@@ -219,7 +221,7 @@ __global__ __launch_bounds__(256) void ragged_conv_kernel(int64_t T, int C, int 
         const int start = seq_off[s];
         const int local = (int)(t - start);
         const float* st = state + (int64_t)slot[s] * (taps - 1) * C;
-        float acc = 0.f;
+        float acc = bias ? bias[c] : 0.f;
         for (int j = 0; j < taps; ++j) {
             const int sl = local - (taps - 1) + j;
             const float in = sl >= 0 ? ldr_dt(x, x_dt, (int64_t)(start + sl) * ldx + c) : st[(int64_t)(taps - 1 + sl) * C + c];
@@ -236,7 +238,8 @@ __global__ __launch_bounds__(256) void ragged_conv_kernel(int64_t T, int C, int 
 template <int TAPS>
 __global__ __launch_bounds__(256) void ragged_conv_vec_kernel(int C, int taps, const void* __restrict__ x, int x_dt, int64_t ldx, const float* __restrict__ w,
                                                               const int* __restrict__ row_seq, const int* __restrict__ seq_off, const int* __restrict__ slot,
-                                                              const float* __restrict__ state, int act, int residual, void* __restrict__ y, int y_dt, int64_t ldy) {
+                                                              const float* __restrict__ state, int act, int residual, void* __restrict__ y, int y_dt, int64_t ldy,
+                                                              const float* __restrict__ bias) {
     const int64_t t = blockIdx.x;
     const int c = 4 * (blockIdx.y * 256 + threadIdx.x);
     if (c >= C) return;
@@ -245,6 +248,7 @@ __global__ __launch_bounds__(256) void ragged_conv_vec_kernel(int C, int taps, c
     const int local = (int)(t - start);
     const float* st = state + (int64_t)slot[s] * (taps - 1) * C;
     f32x4 acc = {0.f, 0.f, 0.f, 0.f}, cur = {0.f, 0.f, 0.f, 0.f};
+    if (bias) acc = *(const f32x4*)(bias + c);
     if constexpr (TAPS > 0) {
         float wf[4 * TAPS];
 #pragma unroll
@@ -301,26 +305,26 @@ __global__ __launch_bounds__(256) void ragged_conv_state_kernel(int n_seq, int C
 }
 
 extern "C" int mi355_ragged_conv(int64_t tokens, int n_seq, int C, int taps, const void* x, int x_dt, int64_t ldx, const float* w, const int* row_seq, const int* seq_off,
-                                 const int* slot, float* state, int act, int residual, void* y, int y_dt, int64_t ldy, void* stream) {
+                                 const int* slot, float* state, int act, int residual, void* y, int y_dt, int64_t ldy, const float* bias, void* stream) {
     MI355_REQUIRE(tokens > 0 && n_seq > 0 && C > 0 && taps >= 1 && taps <= CONV_MAX_TAPS && x && w && row_seq && seq_off && slot && y && (taps == 1 || state),
                   "ragged_conv: bad arguments (taps <= 16)");
     MI355_REQUIRE(rec_dt_ok(x_dt) && rec_dt_ok(y_dt) && ldx >= C && ldy >= C && (act == 0 || act == 1), "ragged_conv: bad operands");
     const int64_t total = tokens * C;
-    if (C % 4 == 0 && ldx % 4 == 0 && ldy % 4 == 0 && al16(x) && al16(y) && al16(state) && tokens < ((int64_t)1 << 31)) {
+    if (C % 4 == 0 && ldx % 4 == 0 && ldy % 4 == 0 && al16(x) && al16(y) && al16(state) && al16(bias) && tokens < ((int64_t)1 << 31)) {
         const dim3 grid((unsigned)tokens, (C / 4 + 255) / 256);
 #define CONV_CASE(TP)                                                                                                                                          \
     case TP:                                                                                                                                                   \
-        ragged_conv_vec_kernel<TP><<<grid, 256, 0, ST(stream)>>>(C, taps, x, x_dt, ldx, w, row_seq, seq_off, slot, state, act, residual, y, y_dt, ldy);      \
+        ragged_conv_vec_kernel<TP><<<grid, 256, 0, ST(stream)>>>(C, taps, x, x_dt, ldx, w, row_seq, seq_off, slot, state, act, residual, y, y_dt, ldy, bias);      \
         break;
         switch (al16(w) ? taps : 0) {
             CONV_CASE(2) CONV_CASE(3) CONV_CASE(4) CONV_CASE(5) CONV_CASE(6) CONV_CASE(7) CONV_CASE(8)
             default:
-                ragged_conv_vec_kernel<0><<<grid, 256, 0, ST(stream)>>>(C, taps, x, x_dt, ldx, w, row_seq, seq_off, slot, state, act, residual, y, y_dt, ldy);
+                ragged_conv_vec_kernel<0><<<grid, 256, 0, ST(stream)>>>(C, taps, x, x_dt, ldx, w, row_seq, seq_off, slot, state, act, residual, y, y_dt, ldy, bias);
         }
 #undef CONV_CASE
     } else {
         const int g = (int)((total + 255) / 256 > 65535 * 8 ? 65535 * 8 : (total + 255) / 256);
-        ragged_conv_kernel<<<g, 256, 0, ST(stream)>>>(tokens, C, taps, x, x_dt, ldx, w, row_seq, seq_off, slot, state, act, residual, y, y_dt, ldy);
+        ragged_conv_kernel<<<g, 256, 0, ST(stream)>>>(tokens, C, taps, x, x_dt, ldx, w, row_seq, seq_off, slot, state, act, residual, y, y_dt, ldy, bias);
     }
     MI355_LAUNCH_CHECK("ragged_conv");
     if (taps > 1) {
@@ -580,7 +584,7 @@ extern "C" int mi355_delta_rule_ragged(int64_t tokens, int n_seq, const int* seq
 
 // ------------------------------------------------------------------------------------------- gated feed-forward activations
 // in[r] = [gate (F) | up (F)] -> out[r, i] (F wide).  kind 0: gelu_tanh(gate) * up.  kind 1: g = min(gate, limit), u = clamp(up, -limit, limit),
-// out = g * sigmoid(1.702 g) * (u + 1).
+// out = g * sigmoid(1.702 g) * (u + 1).  kind 2: silu(gate) * up.
 __global__ __launch_bounds__(256) void glu_rows_kernel(int64_t R, int F, const void* __restrict__ in, int in_dt, int64_t ldi, int kind, float limit, void* __restrict__ out,
                                                        int out_dt, int64_t ldo) {
     const int64_t total = R * F;
@@ -590,6 +594,8 @@ __global__ __launch_bounds__(256) void glu_rows_kernel(int64_t R, int F, const v
         float g = ldr_dt(in, in_dt, r * ldi + i), u = ldr_dt(in, in_dt, r * ldi + F + i), o;
         if (kind == 0) {
             o = 0.5f * g * (1.0f + tanhf(0.7978845608028654f * (g + 0.044715f * g * g * g))) * u;
+        } else if (kind == 2) {
+            o = g / (1.0f + expf(-g)) * u;
         } else {
             g = fminf(g, limit);
             u = fminf(fmaxf(u, -limit), limit);
@@ -613,6 +619,8 @@ __global__ __launch_bounds__(256) void glu_rows_vec_kernel(int64_t R, int F, con
             float g = g4[q], u = u4[q];
             if (kind == 0) {
                 o[q] = 0.5f * g * (1.0f + tanhf(0.7978845608028654f * (g + 0.044715f * g * g * g))) * u;
+            } else if (kind == 2) {
+                o[q] = g / (1.0f + expf(-g)) * u;
             } else {
                 g = fminf(g, limit);
                 u = fminf(fmaxf(u, -limit), limit);
@@ -624,7 +632,7 @@ __global__ __launch_bounds__(256) void glu_rows_vec_kernel(int64_t R, int F, con
 }
 
 extern "C" int mi355_glu_rows(int64_t rows, int F, const void* in, int in_dt, int64_t ld_in, int kind, float limit, void* out, int out_dt, int64_t ld_out, void* stream) {
-    MI355_REQUIRE(rows > 0 && F > 0 && in && out && rec_dt_ok(in_dt) && rec_dt_ok(out_dt) && ld_in >= 2 * (int64_t)F && ld_out >= F && (kind == 0 || kind == 1), "glu_rows: bad arguments");
+    MI355_REQUIRE(rows > 0 && F > 0 && in && out && rec_dt_ok(in_dt) && rec_dt_ok(out_dt) && ld_in >= 2 * (int64_t)F && ld_out >= F && kind >= 0 && kind <= 2, "glu_rows: bad arguments");
     if (F % 4 == 0 && ld_in % 4 == 0 && ld_out % 4 == 0 && al16(in) && al16(out)) {
         const int64_t total4 = rows * (F / 4);
         const int g4 = (int)((total4 + 255) / 256 > 65535 * 8 ? 65535 * 8 : (total4 + 255) / 256);

@@ -175,15 +175,16 @@ def router_logits(x32, w):
 
 
 def moe_route(logits, correction, top, groups, keep, scale, softmax=False):
-    """(ids int32 [tokens, top], weights fp32 [tokens, top]).  ``softmax``: scores are the softmax over all experts, the winners' scores times ``scale`` are
-    the weights (not renormalised); otherwise the grouped sigmoid router."""
+    """(ids int32 [tokens, top], weights fp32 [tokens, top]).  ``softmax`` True: scores are the softmax over all experts, the winners' scores times ``scale``
+    are the weights (not renormalised); ``softmax`` "chosen": ``correction`` is a bias on the logits, the ``top`` largest win and their weights are the
+    softmax over the winners' logits alone (times ``scale``); otherwise the grouped sigmoid router."""
     L.require_gpu(logits, correction)
     if logits.dtype != F32 or not logits.is_contiguous() or (correction is not None and (correction.dtype != F32 or correction.numel() != logits.shape[1])):
         raise ValueError("moe_route: logits contiguous fp32 [tokens, experts], correction fp32 [experts]")
     T, E = logits.shape
     ids = torch.empty((T, top), dtype=I32, device=logits.device)
     wts = torch.empty((T, top), dtype=F32, device=logits.device)
-    L.call("mi355_moe_route", T, E, top, groups, keep, L.ptr(logits), L.ptr(correction), float(scale), 1 if softmax else 0, L.ptr(ids), L.ptr(wts))
+    L.call("mi355_moe_route", T, E, top, groups, keep, L.ptr(logits), L.ptr(correction), float(scale), 2 if softmax == "chosen" else 1 if softmax else 0, L.ptr(ids), L.ptr(wts))
     return ids, wts
 
 
@@ -246,13 +247,14 @@ def attn_key_splits(n_seq, head_tiles, max_new, hm, max_keys, per_split=256):
 
 
 def latent_attn(q, k1, k2, v, out, H, hm, D1, D2, DV, q_hs, k1_hs, v_hs, o_hs, desc, max_new, scale, max_keys=0, kv_rep=1, window=0, keep_first=0, softcap=0.0,
-                sink=None, pool=0, pooled=None, pool_row0=None):
+                sink=None, pool=0, pooled=None, pool_row0=None, chunk=0):
     """Two-part-key causal attention over a ragged batch.  ``desc`` = (q_row0, n_new, past, k1_row0, k2_row0, v_row0) int32 [n_seq] each.  ``max_keys``
     (the longest sequence's keys, if the caller knows it) lets one-token steps over long caches spread a tile's keys over several workgroups.
     ``kv_rep``: query heads per key / value head (strides per key / value head).  ``window`` > 0: a query sees a key only ``window`` positions back, or
     among the first ``keep_first`` of the sequence.  ``softcap`` > 0: scores pass cap * tanh(score / cap).  ``sink`` (fp32 [H]): exp(sink[h]) joins head h's
     denominator.  ``pool`` > 0: ``pooled`` = (pooled keys, pooled values), views laid out like ``k1`` / ``v`` with one mean row per ``pool`` tokens, first row
-    of every sequence in ``pool_row0`` (int32 [n_seq]); a query sees the blocks that lie wholly before its window."""
+    of every sequence in ``pool_row0`` (int32 [n_seq]); a query sees the blocks that lie wholly before its window.  ``chunk`` > 0: positions are cut into chunks
+    of that many from the sequence's first token on, and a query sees only the keys of its own chunk."""
     L.require_gpu(q, k1, k2, v, out, sink, pool_row0, *desc)
     pk = pv = None
     if pool:
@@ -277,11 +279,14 @@ def latent_attn(q, k1, k2, v, out, H, hm, D1, D2, DV, q_hs, k1_hs, v_hs, o_hs, d
     # A plain window leaves a tile window + its own tokens to see: that range is dealt out, in finer shares (a one-token step over it is a chain of
     # dependent 64-key steps in very few workgroups).  A window that also keeps the first tokens is not dealt out: the kernel skips what lies between.
     plain_window = window and window < max_keys and not keep_first
+    reach = min(window or chunk, chunk or window)  # the most keys a row sees besides those of its own tile
+    if chunk and chunk < max_keys and not keep_first:
+        plain_window = True
     if mfma and D1 + D2 <= 320 and DV <= 256 and max_keys and (not window or window >= max_keys or plain_window):
         head_tiles = -(-H // hm)
         tile_tokens = min(max_new, -(-128 // hm))
         if plain_window:  # what a tile walks: its window, and one pooled row per block before it
-            rows = min(max_keys, window + tile_tokens - 1) + (max(0, max_keys - window) // pool if pool else 0)
+            rows = min(max_keys, reach + tile_tokens - 1) + (max(0, max_keys - window) // pool if pool else 0)
             splits = attn_key_splits(n_seq, head_tiles, max_new, hm, rows, 128)
         else:
             splits = attn_key_splits(n_seq, head_tiles, max_new, hm, max_keys)
@@ -291,7 +296,7 @@ def latent_attn(q, k1, k2, v, out, H, hm, D1, D2, DV, q_hs, k1_hs, v_hs, o_hs, d
     L.call("mi355_latent_attn", n_seq, max_new, H, hm, D1, D2, DV, L.ptr(q), q.stride(0), q_hs, L.ptr(k1), k1.stride(0), k1_hs, L.ptr(k2), 0 if k2 is None else k2.stride(0),
            L.ptr(v), v.stride(0), v_hs, L.ptr(out), out.stride(0), o_hs, _dt(v), *[L.ptr(t) for t in desc], float(scale), 1 if mfma else 0, splits, L.ptr(ws),
            0 if ws is None else ws.numel(), int(kv_rep), int(window), int(keep_first), float(softcap or 0.0), L.ptr(sink), int(pool), L.ptr(pk), L.ptr(pv),
-           0 if pk is None else pk.stride(0), L.ptr(pool_row0))
+           0 if pk is None else pk.stride(0), L.ptr(pool_row0), int(chunk))
     return out
 
 
@@ -329,10 +334,12 @@ def group_rmsnorm_sum(x, groups, eps, y1=None, y2=None, parts=1, x_out=None, nor
     return x_out, outs[0], outs[1]
 
 
-def ragged_conv(x, w, state, row_seq, seq_off, slot, act=False, residual=False, out_dtype=None):
+def ragged_conv(x, w, state, row_seq, seq_off, slot, act=False, residual=False, out_dtype=None, bias=None):
     """Causal convolution over time on every channel of the packed rows ``x`` [tokens, C], w fp32 [C, taps]; ``state`` fp32 [slots, taps - 1, C] carries a
-    sequence's last inputs from step to step (read, then updated).  y = (x if residual) + (silu if act)(conv)."""
-    L.require_gpu(x, w, state, row_seq, seq_off, slot)
+    sequence's last inputs from step to step (read, then updated).  y = (x if residual) + (silu if act)(conv + bias)."""
+    L.require_gpu(x, w, state, row_seq, seq_off, slot, bias)
+    if bias is not None and (bias.dtype != F32 or not bias.is_contiguous() or bias.numel() != x.shape[1]):
+        raise ValueError("ragged_conv: bias contiguous fp32 [C]")
     _rows(x, "ragged_conv(x)")
     T, C = x.shape
     taps = w.shape[1]
@@ -346,7 +353,7 @@ def ragged_conv(x, w, state, row_seq, seq_off, slot, act=False, residual=False, 
     _i32(slot, "ragged_conv(slot)")
     y = torch.empty((T, C), dtype=out_dtype or x.dtype, device=x.device)
     L.call("mi355_ragged_conv", T, n_seq, C, taps, L.ptr(x), _dt(x), x.stride(0), L.ptr(w), L.ptr(row_seq), L.ptr(seq_off), L.ptr(slot), L.ptr(state), 1 if act else 0,
-           1 if residual else 0, L.ptr(y), _dt(y), y.stride(0))
+           1 if residual else 0, L.ptr(y), _dt(y), y.stride(0), L.ptr(bias))
     return y
 
 
@@ -404,8 +411,8 @@ def delta_rule(q, k, v, b, a, A_log, dt_bias, qscale, seq_off, slot, state, H, G
     return o
 
 
-GLU_GELU_TANH, GLU_CLAMPED_SWISH = 0, 1
-EPI_RELU2, EPI_CLAMPED_SWISH_GLU, EPI_GELU_TANH_GLU = 1, 2, 3  # epilogues of bgemm
+GLU_GELU_TANH, GLU_CLAMPED_SWISH, GLU_SILU = 0, 1, 2
+EPI_RELU2, EPI_CLAMPED_SWISH_GLU, EPI_GELU_TANH_GLU, EPI_SILU_GLU = 1, 2, 3, 4  # epilogues of bgemm
 
 
 def pack_gate_up(gate, up):
@@ -423,7 +430,8 @@ def pack_gate_up(gate, up):
 
 
 def glu_rows(x, kind, limit=0.0, out_dtype=None):
-    """Rows [gate | up] -> act(gate) * up: ``GLU_GELU_TANH``, or ``GLU_CLAMPED_SWISH`` (g = min(gate, limit), u = clamp(up, +-limit), g sigmoid(1.702 g) (u + 1))."""
+    """Rows [gate | up] -> act(gate) * up: ``GLU_GELU_TANH``, ``GLU_SILU``, or ``GLU_CLAMPED_SWISH`` (g = min(gate, limit), u = clamp(up, +-limit),
+    g sigmoid(1.702 g) (u + 1))."""
     L.require_gpu(x)
     _rows(x, "glu_rows(x)")
     F = x.shape[1] // 2
@@ -490,3 +498,173 @@ def act_rows(x, kind, params=None, gate=None, out_dtype=None):
     L.call("mi355_act_rows", x.shape[0], x.shape[1], L.ptr(x), _dt(x), x.stride(0), L.ptr(gate), 0 if gate is None else _dt(gate), 0 if gate is None else gate.stride(0),
            int(kind), L.ptr(params), L.ptr(out), _dt(out), out.stride(0))
     return out
+
+
+def _vec32(t, n, name):
+    if t is not None and (t.dtype != F32 or not t.is_contiguous() or t.numel() != n):
+        raise ValueError(f"{name}: contiguous fp32 [{n}] required")
+
+
+def dyt_sum(x, ya=None, wa=None, ca=1.0, yb=None, wb=None, cb=1.0, y2=None, parts=1, ls=None, eps=0.0, x_out=None, norm=None, out_dtype=None, want32=False):
+    """The residual sum of a pre-norm block with statistic-free norms: y = ca N_a(ya) + cb N_b(yb) + (sum of y2's ``parts`` rows per token), N an RMS norm
+    over the row with the branch's weight (``wa`` / ``wb`` fp32 [width]) where it has one; v = x + ls * y (``ls`` fp32 [width]: the layer scale).  ``x_out``
+    (True: a new tensor, or a tensor, or None) receives v.  ``norm`` = (alpha, weight, bias): tanh(alpha v) weight + bias is returned in ``out_dtype``
+    (and as fp32 with ``want32``).  Returns (x_out or None, normed or None, normed fp32 or None)."""
+    L.require_gpu(x, ya, wa, yb, wb, y2, ls)
+    _rows(x, "dyt_sum(x)")
+    T, width = x.shape
+    if x.dtype != F32 or not x.is_contiguous():
+        raise ValueError("dyt_sum: x contiguous fp32 [tokens, width]")
+    for y, n, rows in ((ya, "ya", T), (yb, "yb", T), (y2, "y2", T * parts)):
+        if y is not None:
+            _rows(y, f"dyt_sum({n})")
+            if tuple(y.shape) != (rows, width):
+                raise ValueError(f"dyt_sum({n}): [{rows}, {width}] required, got {tuple(y.shape)}")
+    for v, n in ((wa, "wa"), (wb, "wb"), (ls, "ls")):
+        _vec32(v, width, f"dyt_sum({n})")
+    if x_out is True:
+        x_out = torch.empty_like(x)
+    out = out32 = None
+    alpha, w, b = 0.0, None, None
+    if norm is not None:
+        alpha, w, b = norm
+        L.require_gpu(x, w, b)
+        _vec32(w, width, "dyt_sum(weight)")
+        _vec32(b, width, "dyt_sum(bias)")
+        od = out_dtype or F32
+        out = torch.empty((T, width), dtype=od, device=x.device)
+        out32 = out if od == F32 else (torch.empty((T, width), dtype=F32, device=x.device) if want32 else None)
+    L.call("mi355_dyt_sum", T, width, L.ptr(x), L.ptr(ya), 0 if ya is None else _dt(ya), 0 if ya is None else ya.stride(0), L.ptr(wa), float(ca), L.ptr(yb),
+           0 if yb is None else _dt(yb), 0 if yb is None else yb.stride(0), L.ptr(wb), float(cb), L.ptr(y2), 0 if y2 is None else _dt(y2), 0 if y2 is None else y2.stride(0),
+           int(parts), L.ptr(ls), float(eps), L.ptr(x_out), float(alpha), L.ptr(w), L.ptr(b), L.ptr(out), 0 if out is None else _dt(out), None if out32 is out else L.ptr(out32))
+    return x_out, out, out32
+
+
+def token_shift(h, mu, state, row_seq, seq_off, slot, out_dtype):
+    """h fp32 [tokens, C], mu fp32 [n_mix, C] -> [tokens, n_mix * C]: blend s of a row is h + (h' - h) mu[s], h' the sequence's previous row (``state`` fp32
+    [slots, C] before the step's first one; read, then set to the step's last row)."""
+    L.require_gpu(h, mu, state, row_seq, seq_off, slot)
+    _rows(h, "token_shift(h)")
+    T, C = h.shape
+    n_seq = slot.numel()
+    if h.dtype != F32 or mu.dtype != F32 or not mu.is_contiguous() or mu.dim() != 2 or mu.shape[1] != C:
+        raise ValueError("token_shift: h fp32 rows, mu contiguous fp32 [n_mix, C]")
+    if state.dtype != F32 or not state.is_contiguous() or tuple(state.shape[1:]) != (C,):
+        raise ValueError("token_shift: state contiguous fp32 [slots, C]")
+    _i32(row_seq, "token_shift(row_seq)", T)
+    _i32(seq_off, "token_shift(seq_off)", n_seq + 1)
+    _i32(slot, "token_shift(slot)")
+    out = torch.empty((T, mu.shape[0] * C), dtype=out_dtype, device=h.device)
+    L.call("mi355_token_shift", T, n_seq, C, mu.shape[0], L.ptr(h), h.stride(0), L.ptr(mu), L.ptr(row_seq), L.ptr(seq_off), L.ptr(slot), L.ptr(state), L.ptr(out), _dt(out),
+           out.stride(0))
+    return out
+
+
+def _linrec(q, k, v, z, post, u, dt_bias, A_log, D, seq_off, slot, state, H, qk_rep, dk, dv):
+    L.require_gpu(q, k, v, z, u, dt_bias, A_log, D, seq_off, slot, state)
+    T = q.shape[0]
+    G = H // qk_rep
+    for t, n, w in ((q, "q", G * dk), (k, "k", G * dk), (v, "v", H * dv), (z, "z", H if post else H * dk)):
+        _rows(t, f"linrec({n})")
+        if tuple(t.shape) != (T, w):
+            raise ValueError(f"linrec({n}): [{T}, {w}] required, got {tuple(t.shape)}")
+    if q.dtype != k.dtype or z.dtype != F32:
+        raise ValueError("linrec: q / k share a dtype; the decay rows are fp32")
+    n_seq = slot.numel()
+    _i32(seq_off, "linrec(seq_off)", n_seq + 1)
+    _i32(slot, "linrec(slot)")
+    if state.dtype != F32 or not state.is_contiguous() or tuple(state.shape[1:]) != (H, dk, dv):
+        raise ValueError("linrec: state fp32 [slots, H, dk, dv]")
+    o = torch.empty((T, H * dv), dtype=F32, device=q.device)
+    L.call("mi355_linrec_ragged", n_seq, L.ptr(seq_off), L.ptr(slot), H, qk_rep, dk, dv, L.ptr(q), L.ptr(k), _dt(q), q.stride(0), k.stride(0), L.ptr(v), _dt(v), v.stride(0),
+           L.ptr(z), z.stride(0), 1 if post else 0, L.ptr(u), L.ptr(dt_bias), L.ptr(A_log), L.ptr(D), L.ptr(state), L.ptr(o))
+    return o
+
+
+def decay_bonus_attention(r, k, v, z, u, seq_off, slot, state, H, dk, dv):
+    """Linear attention that reads, then updates: o_t = S^T r_t + (sum_i r_i u_i k_i) v_t; S <- diag(exp(-exp(z_t))) S + k_t v_t^T.  z fp32 [tokens, H * dk],
+    u fp32 [H * dk], ``state`` fp32 [slots, H, dk, dv].  Returns fp32 [tokens, H * dv]."""
+    _vec32(u, H * dk, "decay_bonus_attention(u)")
+    return _linrec(r, k, v, z, False, u, None, None, None, seq_off, slot, state, H, 1, dk, dv)
+
+
+def ssd(c, b, x, dt, dt_bias, A_log, D, seq_off, slot, state, H, G, N, P):
+    """State-space duality: per head (group h // (H / G) of b / c) dt = softplus(dt + dt_bias); S <- exp(-exp(A_log) dt) S + b_t (dt x_t)^T;
+    y_t = S^T c_t + D x_t.  b, c [tokens, G * N], x [tokens, H * P], dt fp32 [tokens, H]; ``state`` fp32 [slots, H, N, P].  Returns fp32 [tokens, H * P]."""
+    for t, n in ((dt_bias, "dt_bias"), (A_log, "A_log"), (D, "D")):
+        _vec32(t, H, f"ssd({n})")
+    if H % G:
+        raise ValueError("ssd: heads must be a multiple of groups")
+    return _linrec(c, b, x, dt, True, None, dt_bias, A_log, D, seq_off, slot, state, H, H // G, N, P)
+
+
+def rglru(u, gates, gbias, lam, y, blocks, seq_off, slot, state, out_dtype, decay_c=8.0):
+    """Real-gated linear recurrent unit over a ragged batch: u fp32 [tokens, C], gates fp32 [tokens, 2 C] (per block [recurrence gate | input gate]
+    pre-activations, ``gbias`` fp32 [2 C] their biases or None), lam fp32 [C], y [tokens, C] (the GELU branch before its activation); ``state`` fp32 [slots, C].  Returns S * gelu(y)."""
+    L.require_gpu(u, gates, gbias, lam, y, seq_off, slot, state)
+    for t, n in ((u, "u"), (gates, "gates"), (y, "y")):
+        _rows(t, f"rglru({n})")
+    T, C = u.shape
+    if u.dtype != F32 or gates.dtype != F32 or tuple(gates.shape) != (T, 2 * C) or tuple(y.shape) != (T, C) or C % blocks:
+        raise ValueError("rglru: u fp32 [tokens, C], gates fp32 [tokens, 2 C], y [tokens, C], C a multiple of blocks")
+    _vec32(lam, C, "rglru(lam)")
+    _vec32(gbias, 2 * C, "rglru(gbias)")
+    n_seq = slot.numel()
+    _i32(seq_off, "rglru(seq_off)", n_seq + 1)
+    _i32(slot, "rglru(slot)")
+    if state.dtype != F32 or not state.is_contiguous() or tuple(state.shape[1:]) != (C,):
+        raise ValueError("rglru: state contiguous fp32 [slots, C]")
+    out = torch.empty((T, C), dtype=out_dtype, device=u.device)
+    L.call("mi355_rglru_ragged", n_seq, C, int(blocks), float(decay_c), L.ptr(u), u.stride(0), L.ptr(gates), gates.stride(0), L.ptr(gbias), L.ptr(lam), L.ptr(y), _dt(y), y.stride(0),
+           L.ptr(seq_off), L.ptr(slot), L.ptr(state), L.ptr(out), _dt(out), out.stride(0))
+    return out
+
+
+def gated_groupnorm(o, w, gate, groups, eps, out_dtype, gate_first=False):
+    """o fp32 [tokens, n] in ``groups`` equal consecutive groups, w fp32 [n]: o / rms_group(o) * w * silu(gate), or -- ``gate_first`` -- the RMS norm of
+    o * silu(gate) times w."""
+    L.require_gpu(o, w, gate)
+    _rows(o, "gated_groupnorm(o)")
+    _rows(gate, "gated_groupnorm(gate)")
+    T, n = o.shape
+    if o.dtype != F32 or gate.shape != o.shape or n % groups:
+        raise ValueError("gated_groupnorm: o fp32 [tokens, n], gate of that shape, n a multiple of groups")
+    _vec32(w, n, "gated_groupnorm(w)")
+    out = torch.empty((T, n), dtype=out_dtype, device=o.device)
+    L.call("mi355_gated_groupnorm", T, n, int(groups), L.ptr(o), o.stride(0), L.ptr(w), L.ptr(gate), _dt(gate), gate.stride(0), 1 if gate_first else 0, float(eps), L.ptr(out),
+           _dt(out), out.stride(0))
+    return out
+
+
+UNARY_RELU2, UNARY_TANH, UNARY_HEAD_GATE = 0, 1, 2
+
+
+def unary_rows(x, kind, gate=None, group=1, out_dtype=None):
+    """``UNARY_RELU2``: relu(x)^2; ``UNARY_TANH``; ``UNARY_HEAD_GATE``: x[r, i] * sigmoid(gate[r, i // group]) (gate [rows, n / group])."""
+    L.require_gpu(x, gate)
+    _rows(x, "unary_rows(x)")
+    if kind == UNARY_HEAD_GATE:
+        _rows(gate, "unary_rows(gate)")
+        if x.shape[1] % group or tuple(gate.shape) != (x.shape[0], x.shape[1] // group):
+            raise ValueError("unary_rows: one gate per run of `group` entries")
+    out = torch.empty(x.shape, dtype=out_dtype or x.dtype, device=x.device)
+    L.call("mi355_unary_rows", x.shape[0], x.shape[1], L.ptr(x), _dt(x), x.stride(0), int(kind), L.ptr(gate), 0 if gate is None else _dt(gate),
+           0 if gate is None else gate.stride(0), int(group), L.ptr(out), _dt(out), out.stride(0))
+    return out
+
+
+def scaled_rope_frequencies(dims, base, scaling, device):
+    """fp32 [dims / 2]: base^(-2i / dims), rescaled for a longer context than the one trained on (``scaling`` = {factor, low, high, original}, or None):
+    a frequency whose wavelength is shorter than original / high stays, one longer than original / low is divided by factor, between the two the
+    frequency is blended linearly in original / wavelength.  Evaluated in double."""
+    import math
+
+    i = torch.arange(dims // 2, dtype=torch.float64)
+    f = torch.pow(torch.tensor(float(base), dtype=torch.float64), -2.0 * i / dims)
+    if scaling:
+        fac, lo, hi, orig = (float(scaling[k]) for k in ("factor", "low", "high", "original"))
+        wl = 2.0 * math.pi / f
+        smooth = (orig / wl - lo) / (hi - lo) if hi != lo else torch.ones_like(f)
+        mid = (1.0 - smooth) * f / fac + smooth * f
+        f = torch.where(wl < orig / hi, f, torch.where(wl > orig / lo, f / fac, mid))
+    return f.to(F32).to(device)

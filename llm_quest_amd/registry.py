@@ -40,9 +40,16 @@ def _mopalorn(model_dir, act_dtype, device):
     return load_mopalorn(model_dir, act_dtype, device)
 
 
+def _gepilix(model_dir, act_dtype, device):
+    from llm_quest_amd.gepilix.gepilix_weight_loading import load_gepilix
+
+    return load_gepilix(model_dir, act_dtype, device)
+
+
 register("Gemepel", _gemepel)
 register("Mepatar", _mepatar)
 register("Mopalorn", _mopalorn)
+register("Gepilix", _gepilix)
 
 
 def load_model(model_dir, dtype="bfloat16", device="cuda"):
