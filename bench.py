@@ -539,7 +539,7 @@ def main():
     ap.add_argument("--fp32-tower-leg", choices=["on", "off"], default="on", help="N = 1: also time the same steps with the frozen tower at the reference's fp32 precision (`with_fp32_tower`)")
     ap.add_argument("--other-configs", choices=["on", "off"], default="on", help="N = 1, default batch: append BASELINE configs 2 / 3 / 5 (5 steps each, child processes) as `other_configs`")
     ap.add_argument("--serve", default=None, metavar="MODEL", help="instead of the training step: serving throughput (prompts and one-token steps, random weights) of a registry "
-                    "model -- `gemepel` or `mepatar` beside the Qwen3.5 hybrid text stack, `mopalorn` beside a Mepatar stack of attention layers -- at equal width and depth (llm_quest_amd/serve_bench.py); --steps / --warmup count one-token steps")
+                    "model -- `gemepel` or `mepatar` beside the Qwen3.5 hybrid text stack, `mopalorn` beside a Mepatar stack of attention layers, `gepilix` beside the Mepatar hybrid -- at equal width and depth (llm_quest_amd/serve_bench.py); --steps / --warmup count one-token steps")
     ap.add_argument("--serve-sizes", default="1024x8,2048x16", help="--serve: width x attention heads, comma separated")
     ap.add_argument("--serve-only", action="store_true", help="--serve: skip the reference model's rows")
     args = ap.parse_args()

@@ -261,8 +261,9 @@ def router_choice(h, w, p, mlp):
     return idx[:, :top], gap
 
 
-def forward(cfg, weights, tokens, dtype=torch.float32, return_layers=False):
-    """Logits [T, vocab] of one whole sequence (and the residual stream after every layer)."""
+def forward(cfg, weights, tokens, dtype=torch.float32, return_layers=False, gaps=None):
+    """Logits [T, vocab] of one whole sequence (and the residual stream after every layer).  ``gaps`` (a list) collects, per routed layer, every token's
+    gap between the last chosen and the first rejected router logit."""
     w = {k: (v.to(dtype) if v.is_floating_point() else v) for k, v in weights.items()}
     eps = cfg["norm"]["eps"]
     x = w["embed"][torch.as_tensor(tokens, dtype=torch.long)]
@@ -277,6 +278,8 @@ def forward(cfg, weights, tokens, dtype=torch.float32, return_layers=False):
         if mlp is not None:
             h = dyn_tanh(x, w[p + "norm2.alpha"], w[p + "norm2"], w[p + "norm2.b"])
             y = dense_ff(h, w, p + "mlp.") if mlp["kind"] == "dense" else moe_ff(h, w, p + "mlp.", mlp)
+            if gaps is not None and mlp["kind"] == "moe":
+                gaps.append(router_choice(h, w, p + "mlp.", mlp)[1])
             x = x + w[p + "ls2"] * y
         layers.append(x)
     h = dyn_tanh(x, w["final.norm.alpha"], w["final.norm"], w["final.norm.b"])
