@@ -212,10 +212,9 @@ extern "C" int mi355_token_shift(int64_t tokens, int n_seq, int C, int n_mix, co
 // Per head a state S [dk, dv] (fp32, carried per sequence slot).  Query / key head of value head h: h / qk_rep.
 //   POST == false (read, then update; bonus):  o_t = S^T q_t + (sum_i q_i u_i k_i) v_t;  S <- diag(a_t) S + k_t v_t^T,  a_t[i] = exp(-exp(z[t, h, i]))
 //   POST == true  (update, then read; skip):   dt = softplus(z[t, h] + dt_bias[h]);  S <- exp(-exp(A_log[h]) dt) S + k_t (dt v_t)^T;  o_t = S^T q_t + D[h] v_t
-// Block: 64 value columns x RC row chunks of LR_R key channels; a thread keeps LR_R state entries of one column in registers.  Tokens go through in
+// Block: 64 value columns x RC row chunks of LR_R (8 or 16) key channels; a thread keeps LR_R state entries of one column in registers.  Tokens go through in
 // groups of LR_TB: the group's q / k / decay rows are staged in LDS once (the next group's travel from memory meanwhile), partial sums of the row
 // chunks meet in LDS.
-#define LR_R 16
 #define LR_TB 8
 struct LinRecArgs {
     const int *seq_off, *slot;
@@ -229,7 +228,7 @@ struct LinRecArgs {
     float* o;
 };
 
-template <bool POST>
+template <bool POST, int LR_R>
 __global__ void linrec_kernel(LinRecArgs p) {
     extern __shared__ __attribute__((aligned(16))) float smem[];
     const int RC = blockDim.x >> 6, dk = p.dk, dv = p.dv, H = p.H;
@@ -307,22 +306,45 @@ __global__ void linrec_kernel(LinRecArgs p) {
             b = lanes_sum<8>(b);
             if (part == 0 && j < nt) sb[j] = b;
         }
+        const bool full = chunk * LR_R + LR_R <= dk && dk % 4 == 0;
         for (int j = 0; j < nt; ++j) {
             const float vraw = sv[j * 64 + (threadIdx.x & 63)];
             const float vv = POST ? vraw * sb[j] : vraw;
             const float* qa = sq + j * dk + chunk * LR_R;
             const float* ka = sk + j * dk + chunk * LR_R;
             const float* aa = sa + j * dk + chunk * LR_R;
+            const float a1 = POST ? sa[j * dk] : 0.f;  // update-then-read: one decay for all key channels of the head
             float acc = 0.f;
+            if (full) {
 #pragma unroll
-            for (int r = 0; r < LR_R; ++r) {
-                if (chunk * LR_R + r < dk) {
-                    if (POST) {
-                        st[r] = aa[r] * st[r] + ka[r] * vv;
-                        acc += st[r] * qa[r];
+                for (int r4 = 0; r4 < LR_R / 4; ++r4) {
+                    const f32x4 q4 = *(const f32x4*)(qa + 4 * r4), k4 = *(const f32x4*)(ka + 4 * r4);
+                    if constexpr (POST) {
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) {
+                            st[4 * r4 + i] = a1 * st[4 * r4 + i] + k4[i] * vv;
+                            acc += st[4 * r4 + i] * q4[i];
+                        }
                     } else {
-                        acc += st[r] * qa[r];
-                        st[r] = aa[r] * st[r] + ka[r] * vv;
+                        const f32x4 a4 = *(const f32x4*)(aa + 4 * r4);
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) {
+                            acc += st[4 * r4 + i] * q4[i];
+                            st[4 * r4 + i] = a4[i] * st[4 * r4 + i] + k4[i] * vv;
+                        }
+                    }
+                }
+            } else {
+#pragma unroll
+                for (int r = 0; r < LR_R; ++r) {
+                    if (chunk * LR_R + r < dk) {
+                        if (POST) {
+                            st[r] = aa[r] * st[r] + ka[r] * vv;
+                            acc += st[r] * qa[r];
+                        } else {
+                            acc += st[r] * qa[r];
+                            st[r] = aa[r] * st[r] + ka[r] * vv;
+                        }
                     }
                 }
             }
@@ -349,20 +371,24 @@ __global__ void linrec_kernel(LinRecArgs p) {
 extern "C" int mi355_linrec_ragged(int n_seq, const int* seq_off, const int* slot, int H, int qk_rep, int dk, int dv, const void* q, const void* k, int q_dt, int64_t ldq,
                                    int64_t ldk, const void* v, int v_dt, int64_t ldv, const float* z, int64_t ldz, int post, const float* u, const float* dt_bias,
                                    const float* A_log, const float* D, float* state, float* o, void* stream) {
-    MI355_REQUIRE(n_seq > 0 && n_seq <= 65535 && seq_off && slot && H > 0 && H <= 65535 && qk_rep >= 1 && H % qk_rep == 0 && dk > 0 && dk <= 16 * LR_R && dv > 0 && q && k &&
+    MI355_REQUIRE(n_seq > 0 && n_seq <= 65535 && seq_off && slot && H > 0 && H <= 65535 && qk_rep >= 1 && H % qk_rep == 0 && dk > 0 && dk <= 256 && dv > 0 && q && k &&
                       v && z && state && o && par_dt_ok(q_dt) && par_dt_ok(v_dt),
                   "linrec_ragged: bad arguments (key channels per head <= 256)");
     MI355_REQUIRE(post ? (dt_bias && A_log && D && ldz >= H) : (u && ldz >= (int64_t)H * dk), "linrec_ragged: the update-then-read form takes dt_bias, A_log and D, the other one the bonus");
     MI355_REQUIRE(ldq >= (int64_t)(H / qk_rep) * dk && ldk >= (int64_t)(H / qk_rep) * dk && ldv >= (int64_t)H * dv, "linrec_ragged: rows too short");
-    const int RC = (dk + LR_R - 1) / LR_R;
+    // few key channels per head: eight per thread instead of sixteen, twice the waves to hide the chain's latencies behind
+    const int R = dk <= 64 ? 8 : 16;
+    const int RC = (dk + R - 1) / R;
     const size_t lds_bytes = sizeof(float) * ((size_t)3 * LR_TB * dk + (size_t)LR_TB * 64 + (size_t)LR_TB * RC * 64 + LR_TB);
     MI355_REQUIRE(lds_bytes <= 64 * 1024, "linrec_ragged: LDS budget exceeded");
     LinRecArgs p;
     p.seq_off = seq_off, p.slot = slot, p.H = H, p.dk = dk, p.dv = dv, p.qk_rep = qk_rep, p.q = q, p.k = k, p.v = v, p.z = z, p.q_dt = q_dt, p.v_dt = v_dt;
     p.ldq = ldq, p.ldk = ldk, p.ldv = ldv, p.ldz = ldz, p.u = u, p.dt_bias = dt_bias, p.A_log = A_log, p.D = D, p.state = state, p.o = o;
     const dim3 grid(n_seq, H, (dv + 63) / 64);
-    if (post) linrec_kernel<true><<<grid, 64 * RC, lds_bytes, ST(stream)>>>(p);
-    else linrec_kernel<false><<<grid, 64 * RC, lds_bytes, ST(stream)>>>(p);
+    if (post && R == 8) linrec_kernel<true, 8><<<grid, 64 * RC, lds_bytes, ST(stream)>>>(p);
+    else if (post) linrec_kernel<true, 16><<<grid, 64 * RC, lds_bytes, ST(stream)>>>(p);
+    else if (R == 8) linrec_kernel<false, 8><<<grid, 64 * RC, lds_bytes, ST(stream)>>>(p);
+    else linrec_kernel<false, 16><<<grid, 64 * RC, lds_bytes, ST(stream)>>>(p);
     MI355_LAUNCH_CHECK("linrec_ragged");
     return 0;
 }
@@ -371,46 +397,76 @@ extern "C" int mi355_linrec_ragged(int n_seq, const int* seq_off, const int* slo
 // Per channel c (block b = c / n of n = C / blocks channels, j = c % n): r = sigmoid(gates[t, b * 2n + j] + gbias[b * 2n + j]), i = sigmoid(gates[t, b * 2n + n + j]
 // + gbias[b * 2n + n + j]) (gbias fp32 [2 C] in the gates' layout, may be null);
 // log a = -decay_c * r * softplus(lam[c]);  S <- a S + sqrt(1 - a^2) * (i * u[t, c]);  out[t, c] = S * gelu_tanh(y[t, c]).  1 - a^2 = -expm1(2 log a).
-// state fp32 [slots, C].  One thread per (sequence, channel); the rows of four tokens are fetched before they are used.
-__global__ __launch_bounds__(256) void rglru_kernel(int n_seq, int C, int n, float decay_c, const float* __restrict__ u, int64_t ldu, const float* __restrict__ gates, int64_t ldg,
-                                                    const float* __restrict__ gbias, const float* __restrict__ lam, const void* __restrict__ y, int y_dt, int64_t ldy, const int* __restrict__ seq_off,
-                                                    const int* __restrict__ slot, float* __restrict__ state, void* __restrict__ out, int out_dt, int64_t ldo) {
-    const int64_t total = (int64_t)n_seq * C;
-    for (int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; e < total; e += (int64_t)gridDim.x * blockDim.x) {
-        const int s = (int)(e / C), c = (int)(e % C);
-        const int b = c / n, j = c % n;
-        const int64_t gr = (int64_t)b * 2 * n + j, gi = gr + n;
-        const float sp = decay_c * softplus_p(lam[c]);
-        const float br = gbias ? gbias[gr] : 0.f, bi = gbias ? gbias[gi] : 0.f;
-        float S = state[(int64_t)slot[s] * C + c];
-        const int t0 = seq_off[s], t1 = seq_off[s + 1];
-        for (int tb = t0; tb < t1; tb += 4) {
-            float fu[4], fr[4], fi[4], fy[4];
+// state fp32 [slots, C].
+#define RG_TB 8  // tokens per wave and tile
+#define RG_W 8   // waves of a workgroup: a tile is RG_W * RG_TB consecutive tokens of one sequence
+// Workgroup = 64 channels (lanes) x RG_W waves.  The recurrence S <- a S + b is linear in S, so wave w scans its RG_TB tokens of the tile from zero
+// (local values L_q and the running products P_q of the decays), the waves exchange (P, L) of their last token through LDS, every wave folds what
+// lies before it onto the state the tile came in with, and S_q = L_q + P_q * S_in.  The next tile's rows are requested before the current tile's arithmetic.
+__global__ __launch_bounds__(64 * RG_W) void rglru_kernel(int n_seq, int C, int n, float decay_c, const float* __restrict__ u, int64_t ldu, const float* __restrict__ gates,
+                                                          int64_t ldg, const float* __restrict__ gbias, const float* __restrict__ lam, const void* __restrict__ y, int y_dt,
+                                                          int64_t ldy, const int* __restrict__ seq_off, const int* __restrict__ slot, float* __restrict__ state,
+                                                          void* __restrict__ out, int out_dt, int64_t ldo) {
+    __shared__ float sP[RG_W][64], sL[RG_W][64];
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    const int ctiles = (C + 63) / 64;
+    const int s = blockIdx.x / ctiles, c = (blockIdx.x % ctiles) * 64 + lane;
+    const bool ok = c < C;
+    const int cc = ok ? c : 0;
+    const int b = cc / n, j = cc % n;
+    const int64_t gr = (int64_t)b * 2 * n + j, gi = gr + n;
+    const float sp = decay_c * softplus_p(lam[cc]);
+    const float br = gbias ? gbias[gr] : 0.f, bi = gbias ? gbias[gi] : 0.f;
+    float S = state[(int64_t)slot[s] * C + cc];  // the state the tile comes in with (every wave keeps its own copy)
+    const int t0 = seq_off[s], t1 = seq_off[s + 1];
+    float nu[RG_TB], nr[RG_TB], ni[RG_TB], ny[RG_TB];
+    auto fetch = [&](int tb) {
 #pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                const int64_t t = min(tb + q, t1 - 1);
-                fu[q] = u[t * ldu + c], fr[q] = gates[t * ldg + gr], fi[q] = gates[t * ldg + gi], fy[q] = ldp_dt(y, y_dt, t * ldy + c);
-            }
-#pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                if (tb + q < t1) {
-                    const float r = 1.0f / (1.0f + expf(-(fr[q] + br))), g = 1.0f / (1.0f + expf(-(fi[q] + bi)));
-                    const float la = -sp * r;
-                    S = expf(la) * S + sqrtf(-expm1f(2.0f * la)) * (g * fu[q]);
-                    stp_dt(out, out_dt, (int64_t)(tb + q) * ldo + c, S * gelu_val<1>(fy[q]));
-                }
-            }
+        for (int q = 0; q < RG_TB; ++q) {
+            const int64_t t = min(tb + q, t1 - 1);
+            nu[q] = u[t * ldu + cc], nr[q] = gates[t * ldg + gr], ni[q] = gates[t * ldg + gi], ny[q] = ldp_dt(y, y_dt, t * ldy + cc);
         }
-        state[(int64_t)slot[s] * C + c] = S;
+    };
+    if (t0 + w * RG_TB < t1) fetch(t0 + w * RG_TB);
+    for (int tile = t0; tile < t1; tile += RG_W * RG_TB) {
+        const int tb = tile + w * RG_TB;  // this wave's first token
+        float P[RG_TB], L[RG_TB], gv[RG_TB];
+        float pa = 1.f, ls = 0.f;
+#pragma unroll
+        for (int q = 0; q < RG_TB; ++q) {
+            if (tb + q < t1) {
+                const float r = 1.0f / (1.0f + expf(-(nr[q] + br))), g = 1.0f / (1.0f + expf(-(ni[q] + bi)));
+                const float la = -sp * r, av = expf(la);
+                ls = av * ls + sqrtf(-expm1f(2.0f * la)) * (g * nu[q]);
+                pa *= av;
+                gv[q] = gelu_val<1>(ny[q]);
+            }
+            P[q] = pa, L[q] = ls;
+        }
+        if (tb + RG_W * RG_TB < t1) fetch(tb + RG_W * RG_TB);
+        sP[w][lane] = pa, sL[w][lane] = ls;  // a wave whose tokens lie past the sequence's end leaves (1, 0): the identity
+        __syncthreads();
+        float sin = S, send = S;
+#pragma unroll
+        for (int v = 0; v < RG_W; ++v) {
+            send = sP[v][lane] * send + sL[v][lane];
+            if (v + 1 == w) sin = send;
+        }
+#pragma unroll
+        for (int q = 0; q < RG_TB; ++q)
+            if (ok && tb + q < t1) stp_dt(out, out_dt, (int64_t)(tb + q) * ldo + c, (L[q] + P[q] * sin) * gv[q]);
+        S = send;
+        __syncthreads();
     }
+    if (ok && w == 0) state[(int64_t)slot[s] * C + c] = S;
 }
 
 extern "C" int mi355_rglru_ragged(int n_seq, int C, int blocks, float decay_c, const float* u, int64_t ldu, const float* gates, int64_t ldg, const float* gbias, const float* lam,
                                   const void* y, int y_dt, int64_t ldy, const int* seq_off, const int* slot, float* state, void* out, int out_dt, int64_t ldo, void* stream) {
     MI355_REQUIRE(n_seq > 0 && C > 0 && blocks > 0 && C % blocks == 0 && u && gates && lam && y && seq_off && slot && state && out && par_dt_ok(y_dt) && par_dt_ok(out_dt) &&
-                      ldu >= C && ldg >= 2 * (int64_t)C && ldy >= C && ldo >= C,
+                      ldu >= C && ldg >= 2 * (int64_t)C && ldy >= C && ldo >= C && (int64_t)n_seq * ((C + 63) / 64) < ((int64_t)1 << 31),
                   "rglru_ragged: bad arguments");
-    rglru_kernel<<<par_grid((int64_t)n_seq * C, 256, 65535 * 8), 256, 0, ST(stream)>>>(n_seq, C, C / blocks, decay_c, u, ldu, gates, ldg, gbias, lam, y, y_dt, ldy, seq_off, slot, state,
+    rglru_kernel<<<(unsigned)((int64_t)n_seq * ((C + 63) / 64)), 64 * RG_W, 0, ST(stream)>>>(n_seq, C, C / blocks, decay_c, u, ldu, gates, ldg, gbias, lam, y, y_dt, ldy, seq_off, slot, state,
                                                                                        out, out_dt, ldo);
     MI355_LAUNCH_CHECK("rglru_ragged");
     return 0;
