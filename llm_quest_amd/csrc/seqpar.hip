@@ -42,7 +42,7 @@ __device__ __forceinline__ float silu_p(float g) { return g / (1.0f + expf(-g));
 // ------------------------------------------------------------------------------------------- residual sum, branch join, Dynamic-Tanh norm
 // y = ca * N_a(ya[t]) + cb * N_b(yb[t]) + sum_{p < parts} y2[t * parts + p];  N(y) = y / sqrt(mean(y^2) + eps) * w_n if the branch has a norm weight, else y.
 // v = x[t] + ls * y (ls fp32 [width] or absent: 1);  x_out <- v;  out <- tanh(alpha * v) * w + b (dtype out_dt), out32 <- the same in fp32.
-// One wave per row, four elements per lane and trip (VEC) or one.
+// One wave per row.
 struct DytArgs {
     const float* x;
     float* x_out;
@@ -56,94 +56,110 @@ struct DytArgs {
     int out_dt;
 };
 
-template <bool VEC>
+// Rows of fp32 / bf16 words that are 16-byte aligned, NIT trips of 256 entries per wave (width <= 256 NIT): the branch rows stay in registers between the
+// pass that sums their squares and the pass that joins them, and the vectors (layer scale, weights, bias) come as 16-byte words.  NIT == 0: any width, the
+// branch rows are read twice.
+template <int NIT>
+__global__ __launch_bounds__(256) void dyt_sum_vec_kernel(int64_t T, int width, DytArgs p) {
+    const int lane = threadIdx.x & 63;
+    constexpr int NR = NIT > 0 ? NIT : 1;
+    const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
+    auto ssq = [](f32x4 a) { return a[0] * a[0] + a[1] * a[1] + a[2] * a[2] + a[3] * a[3]; };
+    for (int64_t t = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6); t < T; t += (int64_t)gridDim.x * 4) {
+        f32x4 ka[NR], kb[NR];
+        float ra = 1.f, rb = 1.f, sa = 0.f, sb = 0.f;
+        if constexpr (NIT > 0) {
+#pragma unroll
+            for (int it = 0; it < NIT; ++it) {
+                const int i = (it * 64 + lane) * 4;
+                ka[it] = (p.ya && i < width) ? ldp4_dt(p.ya, p.ya_dt, t * p.ldya + i) : zero;
+                kb[it] = (p.yb && i < width) ? ldp4_dt(p.yb, p.yb_dt, t * p.ldyb + i) : zero;
+                sa += ssq(ka[it]), sb += ssq(kb[it]);
+            }
+        } else {
+            for (int i = lane * 4; i < width; i += 256) {
+                if (p.ya && p.wa) sa += ssq(ldp4_dt(p.ya, p.ya_dt, t * p.ldya + i));
+                if (p.yb && p.wb) sb += ssq(ldp4_dt(p.yb, p.yb_dt, t * p.ldyb + i));
+            }
+        }
+        if (p.ya && p.wa) ra = 1.0f / sqrtf(wave_sum(sa) / (float)width + p.eps);
+        if (p.yb && p.wb) rb = 1.0f / sqrtf(wave_sum(sb) / (float)width + p.eps);
+        const bool any = p.ya || p.yb || p.y2;
+        auto finish = [&](int i, f32x4 a, f32x4 bq) {
+            f32x4 v = *(const f32x4*)(p.x + t * width + i), y = zero;
+            if (p.ya) {
+                if (p.wa) a = a * ra * *(const f32x4*)(p.wa + i);
+                y += p.ca * a;
+            }
+            if (p.yb) {
+                if (p.wb) bq = bq * rb * *(const f32x4*)(p.wb + i);
+                y += p.cb * bq;
+            }
+            if (p.y2)
+                for (int q = 0; q < p.parts; ++q) y += ldp4_dt(p.y2, p.y2_dt, (t * p.parts + q) * p.ldy2 + i);
+            if (any) v += p.ls ? *(const f32x4*)(p.ls + i) * y : y;
+            if (p.x_out) *(f32x4*)(p.x_out + t * width + i) = v;
+            if (p.w) {
+                const f32x4 w4 = *(const f32x4*)(p.w + i), b4 = *(const f32x4*)(p.b + i);
+                f32x4 h;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) h[e] = tanhf(p.alpha * v[e]) * w4[e] + b4[e];
+                if (p.out) stp4_dt(p.out, p.out_dt, t * width + i, h);
+                if (p.out32) *(f32x4*)(p.out32 + t * width + i) = h;
+            }
+        };
+        if constexpr (NIT > 0) {
+#pragma unroll
+            for (int it = 0; it < NIT; ++it) {
+                const int i = (it * 64 + lane) * 4;
+                if (i < width) finish(i, ka[it], kb[it]);
+            }
+        } else {
+            for (int i = lane * 4; i < width; i += 256)
+                finish(i, p.ya ? ldp4_dt(p.ya, p.ya_dt, t * p.ldya + i) : zero, p.yb ? ldp4_dt(p.yb, p.yb_dt, t * p.ldyb + i) : zero);
+        }
+    }
+}
+
+// Any alignment, one entry per lane and trip.
 __global__ __launch_bounds__(256) void dyt_sum_kernel(int64_t T, int width, DytArgs p) {
     const int lane = threadIdx.x & 63;
-    constexpr int W = VEC ? 4 : 1;
     for (int64_t t = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6); t < T; t += (int64_t)gridDim.x * 4) {
         float ra = 1.f, rb = 1.f;
         if (p.ya && p.wa) {
             float s = 0.f;
-            for (int i = lane * W; i < width; i += 64 * W) {
-                if constexpr (VEC) {
-                    const f32x4 a = ldp4_dt(p.ya, p.ya_dt, t * p.ldya + i);
-                    s += a[0] * a[0] + a[1] * a[1] + a[2] * a[2] + a[3] * a[3];
-                } else {
-                    const float a = ldp_dt(p.ya, p.ya_dt, t * p.ldya + i);
-                    s += a * a;
-                }
+            for (int i = lane; i < width; i += 64) {
+                const float a = ldp_dt(p.ya, p.ya_dt, t * p.ldya + i);
+                s += a * a;
             }
             ra = 1.0f / sqrtf(wave_sum(s) / (float)width + p.eps);
         }
         if (p.yb && p.wb) {
             float s = 0.f;
-            for (int i = lane * W; i < width; i += 64 * W) {
-                if constexpr (VEC) {
-                    const f32x4 a = ldp4_dt(p.yb, p.yb_dt, t * p.ldyb + i);
-                    s += a[0] * a[0] + a[1] * a[1] + a[2] * a[2] + a[3] * a[3];
-                } else {
-                    const float a = ldp_dt(p.yb, p.yb_dt, t * p.ldyb + i);
-                    s += a * a;
-                }
+            for (int i = lane; i < width; i += 64) {
+                const float a = ldp_dt(p.yb, p.yb_dt, t * p.ldyb + i);
+                s += a * a;
             }
             rb = 1.0f / sqrtf(wave_sum(s) / (float)width + p.eps);
         }
-        for (int i = lane * W; i < width; i += 64 * W) {
-            float v[W], y[W];
-#pragma unroll
-            for (int e = 0; e < W; ++e) y[e] = 0.f;
-            if constexpr (VEC) {
-                const f32x4 xv = *(const f32x4*)(p.x + t * width + i);
-#pragma unroll
-                for (int e = 0; e < W; ++e) v[e] = xv[e];
-                if (p.ya) {
-                    const f32x4 a = ldp4_dt(p.ya, p.ya_dt, t * p.ldya + i);
-#pragma unroll
-                    for (int e = 0; e < W; ++e) y[e] += p.ca * (p.wa ? a[e] * ra * p.wa[i + e] : a[e]);
-                }
-                if (p.yb) {
-                    const f32x4 a = ldp4_dt(p.yb, p.yb_dt, t * p.ldyb + i);
-#pragma unroll
-                    for (int e = 0; e < W; ++e) y[e] += p.cb * (p.wb ? a[e] * rb * p.wb[i + e] : a[e]);
-                }
-                if (p.y2)
-                    for (int q = 0; q < p.parts; ++q) {
-                        const f32x4 a = ldp4_dt(p.y2, p.y2_dt, (t * p.parts + q) * p.ldy2 + i);
-#pragma unroll
-                        for (int e = 0; e < W; ++e) y[e] += a[e];
-                    }
-            } else {
-                v[0] = p.x[t * width + i];
-                if (p.ya) {
-                    const float a = ldp_dt(p.ya, p.ya_dt, t * p.ldya + i);
-                    y[0] += p.ca * (p.wa ? a * ra * p.wa[i] : a);
-                }
-                if (p.yb) {
-                    const float a = ldp_dt(p.yb, p.yb_dt, t * p.ldyb + i);
-                    y[0] += p.cb * (p.wb ? a * rb * p.wb[i] : a);
-                }
-                if (p.y2)
-                    for (int q = 0; q < p.parts; ++q) y[0] += ldp_dt(p.y2, p.y2_dt, (t * p.parts + q) * p.ldy2 + i);
+        for (int i = lane; i < width; i += 64) {
+            float v = p.x[t * width + i], y = 0.f;
+            if (p.ya) {
+                const float a = ldp_dt(p.ya, p.ya_dt, t * p.ldya + i);
+                y += p.ca * (p.wa ? a * ra * p.wa[i] : a);
             }
-            float h[W];
-#pragma unroll
-            for (int e = 0; e < W; ++e) {
-                if (p.ya || p.yb || p.y2) v[e] += p.ls ? p.ls[i + e] * y[e] : y[e];
-                h[e] = p.w ? tanhf(p.alpha * v[e]) * p.w[i + e] + p.b[i + e] : 0.f;
+            if (p.yb) {
+                const float a = ldp_dt(p.yb, p.yb_dt, t * p.ldyb + i);
+                y += p.cb * (p.wb ? a * rb * p.wb[i] : a);
             }
-            if constexpr (VEC) {
-                if (p.x_out) *(f32x4*)(p.x_out + t * width + i) = f32x4{v[0], v[1], v[2], v[3]};
-                if (p.w) {
-                    const f32x4 hv = {h[0], h[1], h[2], h[3]};
-                    if (p.out) stp4_dt(p.out, p.out_dt, t * width + i, hv);
-                    if (p.out32) *(f32x4*)(p.out32 + t * width + i) = hv;
-                }
-            } else {
-                if (p.x_out) p.x_out[t * width + i] = v[0];
-                if (p.w) {
-                    if (p.out) stp_dt(p.out, p.out_dt, t * width + i, h[0]);
-                    if (p.out32) p.out32[t * width + i] = h[0];
-                }
+            if (p.y2)
+                for (int q = 0; q < p.parts; ++q) y += ldp_dt(p.y2, p.y2_dt, (t * p.parts + q) * p.ldy2 + i);
+            if (p.ya || p.yb || p.y2) v += p.ls ? p.ls[i] * y : y;
+            if (p.x_out) p.x_out[t * width + i] = v;
+            if (p.w) {
+                const float h = tanhf(p.alpha * v) * p.w[i] + p.b[i];
+                if (p.out) stp_dt(p.out, p.out_dt, t * width + i, h);
+                if (p.out32) p.out32[t * width + i] = h;
             }
         }
     }
@@ -164,8 +180,12 @@ extern "C" int mi355_dyt_sum(int64_t tokens, int width, const float* x, const vo
     const bool vec = width % 4 == 0 && par_al16(x) && par_al16(x_out) && par_al16(ya) && par_al16(yb) && par_al16(y2) && par_al16(out) && par_al16(out32) && ldya % 4 == 0 &&
                      ldyb % 4 == 0 && ldy2 % 4 == 0 && par_al16(wa) && par_al16(wb) && par_al16(ls) && par_al16(w) && par_al16(b);
     const int grid = par_grid(tokens, 4, 65535 * 16);
-    if (vec) dyt_sum_kernel<true><<<grid, 256, 0, ST(stream)>>>(tokens, width, p);
-    else dyt_sum_kernel<false><<<grid, 256, 0, ST(stream)>>>(tokens, width, p);
+    if (!vec) dyt_sum_kernel<<<grid, 256, 0, ST(stream)>>>(tokens, width, p);
+    else if (width <= 256) dyt_sum_vec_kernel<1><<<grid, 256, 0, ST(stream)>>>(tokens, width, p);
+    else if (width <= 512) dyt_sum_vec_kernel<2><<<grid, 256, 0, ST(stream)>>>(tokens, width, p);
+    else if (width <= 1024) dyt_sum_vec_kernel<4><<<grid, 256, 0, ST(stream)>>>(tokens, width, p);
+    else if (width <= 2048) dyt_sum_vec_kernel<8><<<grid, 256, 0, ST(stream)>>>(tokens, width, p);
+    else dyt_sum_vec_kernel<0><<<grid, 256, 0, ST(stream)>>>(tokens, width, p);
     MI355_LAUNCH_CHECK("dyt_sum");
     return 0;
 }
