@@ -543,16 +543,21 @@ __global__ __launch_bounds__(256) void unary_rows_kernel(int64_t R, int n, const
     }
 }
 template <int KIND>
-__global__ __launch_bounds__(256) void unary_rows_vec_kernel(int64_t R, int n, const void* __restrict__ x, int x_dt, int64_t ldx, void* __restrict__ out, int out_dt,
-                                                             int64_t ldo) {
+__global__ __launch_bounds__(256) void unary_rows_vec_kernel(int64_t R, int n, const void* __restrict__ x, int x_dt, int64_t ldx, const void* __restrict__ gate, int g_dt,
+                                                             int64_t ldg, int group, void* __restrict__ out, int out_dt, int64_t ldo) {
     const int n4 = n / 4;
     const int64_t total = R * n4;
     for (int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; e < total; e += (int64_t)gridDim.x * blockDim.x) {
         const int64_t r = e / n4;
         const int i = 4 * (int)(e % n4);
         f32x4 a = ldp4_dt(x, x_dt, r * ldx + i);
+        if constexpr (KIND == 2) {  // four neighbours share a gate (group is a multiple of 4)
+            const float sg = 1.0f / (1.0f + expf(-ldp_dt(gate, g_dt, r * ldg + i / group)));
+            a = a * sg;
+        } else {
 #pragma unroll
-        for (int q = 0; q < 4; ++q) a[q] = KIND == 0 ? (a[q] > 0.f ? a[q] * a[q] : 0.f) : tanhf(a[q]);
+            for (int q = 0; q < 4; ++q) a[q] = KIND == 0 ? (a[q] > 0.f ? a[q] * a[q] : 0.f) : tanhf(a[q]);
+        }
         stp4_dt(out, out_dt, r * ldo + i, a);
     }
 }
@@ -561,10 +566,11 @@ extern "C" int mi355_unary_rows(int64_t rows, int n, const void* x, int x_dt, in
                                 int out_dt, int64_t ldo, void* stream) {
     MI355_REQUIRE(rows > 0 && n > 0 && x && out && par_dt_ok(x_dt) && par_dt_ok(out_dt) && ldx >= n && ldo >= n && kind >= 0 && kind <= 2, "unary_rows: bad arguments");
     MI355_REQUIRE(kind != 2 || (gate && par_dt_ok(g_dt) && group >= 1 && ldg >= (n + group - 1) / group), "unary_rows: a head gate needs its rows and the head size");
-    if (kind < 2 && n % 4 == 0 && ldx % 4 == 0 && ldo % 4 == 0 && par_al16(x) && par_al16(out)) {
+    if ((kind < 2 || group % 4 == 0) && n % 4 == 0 && ldx % 4 == 0 && ldo % 4 == 0 && par_al16(x) && par_al16(out)) {
         const int g4 = par_grid(rows * (n / 4), 256, 65535 * 8);
-        if (kind == 0) unary_rows_vec_kernel<0><<<g4, 256, 0, ST(stream)>>>(rows, n, x, x_dt, ldx, out, out_dt, ldo);
-        else unary_rows_vec_kernel<1><<<g4, 256, 0, ST(stream)>>>(rows, n, x, x_dt, ldx, out, out_dt, ldo);
+        if (kind == 0) unary_rows_vec_kernel<0><<<g4, 256, 0, ST(stream)>>>(rows, n, x, x_dt, ldx, gate, g_dt, ldg, group, out, out_dt, ldo);
+        else if (kind == 1) unary_rows_vec_kernel<1><<<g4, 256, 0, ST(stream)>>>(rows, n, x, x_dt, ldx, gate, g_dt, ldg, group, out, out_dt, ldo);
+        else unary_rows_vec_kernel<2><<<g4, 256, 0, ST(stream)>>>(rows, n, x, x_dt, ldx, gate, g_dt, ldg, group, out, out_dt, ldo);
         MI355_LAUNCH_CHECK("unary_rows");
         return 0;
     }
