@@ -135,8 +135,8 @@ def gepilix_config(width, heads, vocab=32000):
     rescaled frequencies) beside a state-space layer (heads of 64 filling twice the width, state 128, one group, 4 taps), decay attention again; three layers
     with 16 experts (2 per token, ff = 1.75 width) plus a shared expert of the same size, one dense squared-ReLU layer (ff = 3.5 width)."""
     wkv = {"heads": width // 64, "dim": 64}
-    att = {"heads": heads, "kv_heads": 2, "dim": 128, "vdim": 128, "mask": {"size": 512}, "scale": 128 ** -0.5, "softcap": 30.0}
-    rot = {"dims": 64, "base": 1e6, "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 8192}}
+    att = {"heads": heads, "kv_heads": 2, "dim": 128, "vdim": 128, "mask": {"size": 512}, "scale": 128 ** -0.5, "softcap": 50.0}
+    rot = {"dims": 64, "base": 5e5, "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 8192}}
     moe = {"kind": "moe", "expert": {"ff": int(width * 1.75)}, "router": {"experts": 16, "top": 2}, "shared": {"ff": int(width * 1.75)}}
     dense = {"kind": "dense", "ff": int(width * 3.5)}
     layers = [{"type": "wkv", "mixer": wkv, "mlp": moe},
