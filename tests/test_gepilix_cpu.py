@@ -82,3 +82,23 @@ def test_registry_knows_the_design():
     from llm_quest_amd import registry
 
     assert "Gepilix" in registry.architectures()
+
+
+def test_serving_bench_configuration_parses_beside_its_reference():
+    """The bench's Gepilix model builds at both sizes and stands beside a Mepatar hybrid of about as many weights."""
+    from llm_quest_amd import serve_bench as B
+    from llm_quest_amd.gepilix.gepilix_model import GepilixConfig
+    from llm_quest_amd.mepatar.mepatar_model import MepatarConfig
+
+    for width, heads in ((1024, 8), (2048, 16)):
+        cfg = GepilixConfig(B.gepilix_config(width, heads))
+        assert [l["type"] for l in cfg.layers] == ["wkv", "parallel", "parallel_2", "wkv"] and set(cfg.decay_ranks) == {0, 3}
+        ref = MepatarConfig(B.mepatar_config(width, heads))
+        assert len(ref.layers) == len(cfg.layers) and ref.width == cfg.width
+    with torch.device("meta"):
+        from llm_quest_amd.gepilix.gepilix_model import GepilixModel
+        from llm_quest_amd.mepatar.mepatar_model import MepatarModel
+
+        a = sum(p.numel() for p in GepilixModel(GepilixConfig(B.gepilix_config(1024, 8), {0: 64, 3: 64})).parameters())
+        b = sum(p.numel() for p in MepatarModel(MepatarConfig(B.mepatar_config(1024, 8))).parameters())
+    assert 0.9 < a / b < 1.1
